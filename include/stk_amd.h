@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 8
+#define STK_AMD_ABI_VERSION 9
 
 /* status codes */
 #define STK_OK 0
@@ -148,16 +148,21 @@ int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
  * plan (optional) is the fusion plan of the stored matrix.
  * workspace (optional; no counterpart in the reference; used with a plan only) lets a
  * launch whose tiles would fill the GPU only a few times cut the tiles of its last,
- * partly filled round into slices along k, computed by different workgroups: 256-byte
- * aligned device memory of at least stk_dsd_workspace_bytes(m, n, blocking) bytes (0:
- * this shape never uses one).  Its first 4 * (number of compute units) bytes (counters)
- * must be zero before the first launch that uses it; every launch leaves them zero.
+ * partly filled round into slices along k, computed by different workgroups.  It is
+ * 256-byte aligned device memory: stk_dsd_workspace_counter_bytes() bytes of counters, which
+ * must be zero before the first launch that uses them (every launch that completes leaves
+ * them zero), followed by room for partial tiles of stk_dsd_workspace_slot_bytes() bytes
+ * each.  stk_dsd_workspace_bytes(m, n, blocking) is the size with which no launch of this
+ * shape is limited (0: this shape never uses a workspace); a smaller one is accepted and the
+ * last round is cut into fewer slices, or not at all, so that its partial tiles fit.
  * Launches that may overlap need separate workspaces.  With a workspace the sums over k
  * of the sliced tiles are associated differently (fp32), so results can differ in the
  * last bit from those without; they are the same from run to run.  STK_ERR_WORKSPACE
- * when it is needed and too small or misaligned.
+ * when it is misaligned.
  */
 int64_t stk_dsd_workspace_bytes(int64_t m, int64_t n, int blocking);
+int64_t stk_dsd_workspace_counter_bytes(void);
+int64_t stk_dsd_workspace_slot_bytes(void);
 /*
  * The rule behind the slice counts that stk_build_plan stores for stk_dsd, evaluated on the
  * host (for inspection and tests): into how many slices along k (1 .. 4) the tiles of the last

@@ -11,6 +11,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
+ABI_VERSION = 9
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
 STK_F16, STK_BF16 = 0, 1
 STK_I16, STK_I32 = 0, 1
@@ -26,6 +27,8 @@ SIGNATURES = {
     "stk_sdd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _p]),
     "stk_sdd_fused": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _int, _p, _p]),
     "stk_dsd_workspace_bytes": (_i64, [_i64, _i64, _int]),
+    "stk_dsd_workspace_counter_bytes": (_i64, []),
+    "stk_dsd_workspace_slot_bytes": (_i64, []),
     "stk_dsd_tail_slices": (_int, [_i64, _i64, _i64, ctypes.c_double, _int]),
     "stk_dsd": (_int, [_i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _int, _p, _p, _i64, _p]),
     "stk_dds": (_int, [_i64, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _int, _int, _int, _p, _p]),
@@ -63,7 +66,7 @@ def load():
                 fn = getattr(lib, name)
                 fn.restype = res
                 fn.argtypes = args
-            if lib.stk_abi_version() != 8:
+            if lib.stk_abi_version() != ABI_VERSION:
                 raise RuntimeError("stk_amd: libstk_amd.so has an unexpected ABI version; rebuild it")
             _lib = lib
     return _lib

@@ -74,6 +74,7 @@ def _side_stream(device):
     stream = _side_streams.get(device.index)
     if stream is None:
         stream = _side_streams[device.index] = torch.cuda.Stream(device=device)
+        backend.CONCURRENT_STREAMS.add(stream.cuda_stream)   # its dsd launches get a workspace of their own
     return stream
 
 

@@ -96,18 +96,50 @@ def _validate_matmul_dims(m, k, n, blocking):
 FUSION = True
 
 
+def _version_of(t):
+    """In-place modification counter of a tensor, or None for a tensor that keeps none (inference mode)."""
+    return None if t.is_inference() else t._version
+
+
+def _plan_cache_get(tensors, blocking):
+    """The cache entry on tensors[0] (`offsets`) if it describes exactly these index tensors in their
+    present state, else None.  The entry keeps the other index tensors it was built from: their storage
+    stays alive, so an address cannot come back with other contents, and identity plus the version
+    counters say whether they still hold what the plan describes.  A plan built with the transpose
+    metadata also serves a request without it."""
+    cached = getattr(tensors[0], "_stk_plan", None)
+    if cached is None or cached[2] != blocking or len(cached[0]) < len(tensors) - 1:
+        return None
+    versions = tuple(_version_of(t) for t in tensors)
+    if None in versions or cached[5][:len(versions)] != versions or not all(a is b for a, b in zip(cached[0], tensors[1:])):
+        return None
+    return cached
+
+
+def _plan_cache_put(tensors, blocking, plan, stream_handle, built):
+    """Remembers `plan` on tensors[0]; tensors without a version counter (made under inference mode)
+    cannot be watched for in-place changes and are not cached."""
+    versions = tuple(_version_of(t) for t in tensors)
+    if None in versions:
+        return False
+    try:
+        tensors[0]._stk_plan = (tuple(tensors[1:]), plan, blocking, stream_handle, built, versions)
+    except AttributeError:
+        return False
+    return True
+
+
 def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, blocking=128):
     """Device tensor with the fusion roles of the block rows (and, when the
     transpose metadata is given, of the block columns): which neighbouring lines
     repeat each other and are computed as one 256-wide tile.  Depends on the
     topology only, so it is cached on the `offsets` tensor and rebuilt when one of
-    the index tensors has been modified in place."""
+    the index tensors has been replaced or modified in place."""
     _need_gpu(offsets, column_indices)
     want_cols = offsets_t is not None and column_indices_t is not None
     tensors = (offsets, column_indices) + ((offsets_t, column_indices_t) if want_cols else ())
-    key = tuple((t.data_ptr(), t._version, t.numel()) for t in tensors)
-    cached = getattr(offsets, "_stk_plan", None)
-    if cached is not None and cached[2] == blocking and cached[0][:2] == key[:2] and (not want_cols or cached[0] == key):
+    cached = _plan_cache_get(tensors, blocking)
+    if cached is not None:
         stream = torch.cuda.current_stream(offsets.device)
         if cached[3] != stream.cuda_stream:
             stream.wait_event(cached[4])  # built on another stream: what this one launches next comes after the build
@@ -128,10 +160,7 @@ def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, 
     stream = torch.cuda.current_stream(offsets.device)
     built = torch.cuda.Event()
     built.record(stream)
-    try:
-        offsets._stk_plan = (key, plan, blocking, stream.cuda_stream, built)
-    except AttributeError:
-        pass
+    _plan_cache_put(tensors, blocking, plan, stream.cuda_stream, built)
     return plan
 
 
@@ -190,24 +219,42 @@ def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activa
 # along k, which takes a workspace.  Results then differ in the last bit from the uncut sums;
 # switching it off restores those.
 SLICE_LAST_ROUND = True
-_dsd_workspaces = {}
+# Partial tiles (256 KiB each) the workspace of a device has room for: 256 of them (64 MiB) let a last round of
+# 128 tiles be cut in two, or one of 64 tiles in four; a launch that would like more is cut less.  The buffer is
+# allocated on the first dsd that can use it and kept; release_workspaces() frees it.
+DSD_WORKSPACE_SLOTS = 256
+# Streams whose dsd launches may run beside those of other streams (the autograd layer's side stream): they get
+# a workspace of their own.  Everything else shares one per device, and a launch on another stream than the
+# last one first waits for that stream.
+CONCURRENT_STREAMS = set()
+_dsd_workspaces = {}   # (device index, concurrent lane) -> [buffer, stream of the last launch]
+
+
+def release_workspaces():
+    """Frees the dsd workspaces (they are allocated again on demand)."""
+    _dsd_workspaces.clear()
 
 
 def _dsd_workspace(device, m, n, blocking):
-    """Workspace of stk_dsd for this shape, or None.  One buffer per (device, stream): launches on
-    one stream do not overlap, and every launch leaves the counters at the front zero."""
+    """Workspace of stk_dsd for this shape, or None: [counters | slots], the counters zero between launches."""
     if not SLICE_LAST_ROUND:
         return None
-    nbytes = _lib.load().stk_dsd_workspace_bytes(m, n, blocking)
-    if nbytes <= 0:
+    lib = _lib.load()
+    if lib.stk_dsd_workspace_bytes(m, n, blocking) <= 0:
         return None
-    key = (device.index, _stream())
-    ws = _dsd_workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
+    stream = torch.cuda.current_stream(device)
+    key = (device.index, stream.cuda_stream in CONCURRENT_STREAMS)
+    entry = _dsd_workspaces.get(key)
+    counters = lib.stk_dsd_workspace_counter_bytes()
+    nbytes = counters + DSD_WORKSPACE_SLOTS * lib.stk_dsd_workspace_slot_bytes()
+    if entry is None or entry[0].numel() != nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        ws[:4096].zero_()   # the counters; the slots behind them need no initial value
-        _dsd_workspaces[key] = ws
-    return ws
+        ws[:counters].zero_()   # the slots behind the counters need no initial value
+        entry = _dsd_workspaces[key] = [ws, stream]
+    elif entry[1].cuda_stream != stream.cuda_stream:
+        stream.wait_stream(entry[1])   # launches that share a workspace must not overlap
+        entry[1] = stream
+    return entry[0]
 
 
 def dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,
@@ -226,14 +273,17 @@ def dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_ind
     ci, cit = _index(column_indices), _index(column_indices_t)
     plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t) if FUSION and b == 128 and data.shape[0] > 0 else None
     with _on_device(out.device):
-        ws = _dsd_workspace(out.device, m, n, b)
-        _lib.check(_lib.load().stk_dsd(
+        ws = _dsd_workspace(out.device, m, n, b) if plan is not None else None
+        status = _lib.load().stk_dsd(
             m, k, n, data.data_ptr(), _offsets(offsets).data_ptr(), ci.data_ptr(),
             _offsets(offsets_t).data_ptr(), cit.data_ptr(), _offsets(block_offsets_t).data_ptr(),
             1 if transpose_a else 0, rhs.data_ptr(), rhs.stride(0), rhs.stride(1),
             out.data_ptr(), out.stride(0), data.shape[0], b, _value_dtype(out), _INDEX_DTYPES[ci.dtype],
             plan.data_ptr() if plan is not None else None,
-            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream())
+        if status != _lib.STK_OK and ws is not None:
+            release_workspaces()   # whatever a failed launch left in the counters is not reused
+        _lib.check(status)
 
 
 def dds(lhs, shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,

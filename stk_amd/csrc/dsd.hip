@@ -147,8 +147,9 @@ __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists 
 // ---------------------------------------------------------------------------
 struct TailArgs {
   int32_t* counters;  // one per tile of the last round; zero between launches
-  float* slots;       // kMaxTailSlices per tile of the last round, kSlotFloats each
+  float* slots;       // `slices` per tile of the last round, kSlotFloats each
   int workgroups;     // workgroups per round: the compute units
+  int capacity;       // slots the workspace holds; the last round is cut no further than fits
 };
 constexpr int kSlotFloats = 512 * 128;  // 512 threads x up to 8 accumulators of 16 values
 constexpr int kTailBlock = 32;          // tiles whose slices are interleaved: 4 neighbours on each of the 8 compute dies
@@ -181,12 +182,14 @@ __device__ __forceinline__ void add_slices_in_order(f32x16_t (&acc)[Cfg::IM][Cfg
   }
 }
 
-// Slice `slice` of `slices` of the tile (LINES block rows from bi, columns from n0), the `ordinal`-th tile of the last round.
+// Slice `slice` of `slices` of the tile (LINES block rows from bi, columns from n0), the `ordinal`-th tile of the last
+// round; the tile owns the slots [ordinal * slices, (ordinal + 1) * slices) of the workspace.
 template <class Cfg, bool TRANS_A, int LINES>
 __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, int bi, int n0, int slice, int slices, int ordinal, char* smem, int* flag) {
   constexpr int kAcc = Cfg::IM * Cfg::JN;
   static_assert(kAcc * 16 * 512 <= kSlotFloats, "slot too small");
   const int nseg = g.walk_offsets[bi + 1] - g.walk_offsets[bi];
+  const int64_t first_slot = (int64_t)ordinal * slices;
   if (slices > nseg) slices = nseg > 1 ? nseg : 1;
   if (slice >= slices) return;
   const int e0 = slice * nseg / slices, e1 = (slice + 1) * nseg / slices;
@@ -203,7 +206,7 @@ __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, i
   // holds value r of accumulator a of thread t at (16 a + r) * 512 + t.
   const int others = slices - 1;
   int32_t* counter = t.counters + ordinal;
-  auto slot_of = [&](int sl) { return t.slots + ((int64_t)ordinal * kMaxTailSlices + sl) * kSlotFloats + tid; };
+  auto slot_of = [&](int sl) { return t.slots + (first_slot + sl) * kSlotFloats + tid; };
   if (tid == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   int arrived = uniform(*flag);
@@ -243,7 +246,7 @@ __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, i
     }
   } else {
     // more: always in the order of the slices, whoever does the adding
-    const float* first = t.slots + (int64_t)ordinal * kMaxTailSlices * kSlotFloats + tid;
+    const float* first = slot_of(0);
     switch (slices * kMaxTailSlices + slice) {
       case 3 * kMaxTailSlices + 0: add_slices_in_order<Cfg, 3, 0>(acc, first); break;
       case 3 * kMaxTailSlices + 1: add_slices_in_order<Cfg, 3, 1>(acc, first); break;
@@ -272,7 +275,12 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   if (slices < 1 || slices > kMaxTailSlices) slices = 1;
   // whole rounds first; the rest (all of it when there is less than one round) is the last round
-  const int whole = (slices > 1 && tiles > 0) ? (tiles - 1) / t.workgroups * t.workgroups : tiles;
+  int whole = (slices > 1 && tiles > 0) ? (tiles - 1) / t.workgroups * t.workgroups : tiles;
+  if (slices > 1 && (tiles - whole) * slices > t.capacity) {
+    // a workspace smaller than the plan would like: fewer slices, or none
+    slices = t.capacity / (tiles - whole);
+    if (slices < 2) slices = 1, whole = tiles;
+  }
   int item = blockIdx.x, slice = 0;
   if (item >= whole) {
     // last round: blocks of kTailBlock tiles, slice by slice, so that neighbouring tiles (which share
@@ -419,13 +427,15 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
   if (workspace && plan && blocking == 128 && n % 256 == 0 && nnz > 0 && !g.small) {
     const int workgroups = compute_units();
     if (workgroups > 0 && block_rows * (n / 128) / 3 < 8 * (int64_t)workgroups) {
-      const size_t need = tail_workspace_bytes(workgroups);
-      if ((size_t)workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-        return fail(STK_ERR_WORKSPACE, "stk_dsd: workspace of %lld bytes (256-byte aligned) needed, %lld given", (long long)need, (long long)workspace_bytes);
-      sliced = true;
-      tail.counters = static_cast<int32_t*>(workspace);
-      tail.slots = reinterpret_cast<float*>(static_cast<char*>(workspace) + tail_counter_bytes(workgroups));
-      tail.workgroups = workgroups;
+      if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(STK_ERR_WORKSPACE, "stk_dsd: the workspace must be 256-byte aligned");
+      const int64_t capacity = (workspace_bytes - (int64_t)tail_counter_bytes(workgroups)) / (int64_t)(sizeof(float) * kSlotFloats);
+      if (capacity >= 2) {
+        sliced = true;
+        tail.counters = static_cast<int32_t*>(workspace);
+        tail.slots = reinterpret_cast<float*>(static_cast<char*>(workspace) + tail_counter_bytes(workgroups));
+        tail.workgroups = workgroups;
+        tail.capacity = (int)(capacity < kMaxTailSlices * (int64_t)workgroups ? capacity : kMaxTailSlices * (int64_t)workgroups);
+      }
     }
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -440,6 +450,13 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
   STK_DSD_LAYOUTS(true, 128) STK_DSD_LAYOUTS(false, 128) STK_DSD_LAYOUTS(true, 64) STK_DSD_LAYOUTS(false, 64)
   return fail(STK_ERR_UNSUPPORTED, "stk_dsd: no kernel for this configuration");
 }
+
+extern "C" int64_t stk_dsd_workspace_counter_bytes(void) {
+  const int workgroups = stk::compute_units();
+  return workgroups > 0 ? (int64_t)stk::tail_counter_bytes(workgroups) : 0;
+}
+
+extern "C" int64_t stk_dsd_workspace_slot_bytes(void) { return (int64_t)(sizeof(float) * stk::kSlotFloats); }
 
 extern "C" int64_t stk_dsd_workspace_bytes(int64_t m, int64_t n, int blocking) {
   using namespace stk;

@@ -1,4 +1,6 @@
 """Shared helpers for the GPU parity tests: seeded inputs, oracle bridges, tolerances."""
+import zlib
+
 import numpy as np
 import torch
 
@@ -6,6 +8,21 @@ from oracle import stk_oracle as O
 
 # north-star tolerances against the fp32 oracle
 TOL = {torch.bfloat16: dict(rtol=1e-2, atol=1e-2), torch.float16: dict(rtol=1e-2, atol=5e-3)}
+
+
+# Scale-free bounds beside them.  The absolute tolerances above exceed the size of the outputs when the
+# operands are ~N(0, 0.02), so a result can lose a whole K-tile and still pass them; these cannot be passed
+# that way.  A result rounded once to 16 bits from an exact sum is off by at most half an ulp, i.e. 2^-8
+# (bfloat16) or 2^-11 (float16) of its own size:
+#   max |got - want|  <=  MAX_REL * max |want|       (2x / 4x half an ulp of the largest element)
+#   ||got - want||_F  <=  RMS_REL * ||want||_F       (rounding noise is about 0.4 x 2^-8 resp. 2^-11 of the norm)
+MAX_REL = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -9}
+RMS_REL = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}
+
+
+def stable_seed(*args):
+    """Seed derived from the arguments that is the same in every process (Python's hash() of strings is not)."""
+    return zlib.crc32(repr(tuple(str(a) for a in args)).encode()) % (2 ** 31)
 
 
 def np32(t):
@@ -30,6 +47,29 @@ def assert_close(got, want, dtype, what=""):
         idx = np.argwhere(bad)[0]
         raise AssertionError(f"{what}: {bad.sum()} of {bad.size} elements outside rtol={tol['rtol']} atol={tol['atol']}; "
                              f"first at {tuple(idx)}: got {got[tuple(idx)]} want {want[tuple(idx)]}")
+
+
+def assert_close_scaled(got, want, dtype, what=""):
+    """The north-star tolerance and the two scale-free bounds, for tensors on any device (computed there,
+    so that full-size results need not travel to the host).  `want` is the fp32 reference."""
+    got = got.detach().float() if isinstance(got, torch.Tensor) else torch.as_tensor(np.asarray(got, dtype=np.float32))
+    want = want.detach().float() if isinstance(want, torch.Tensor) else torch.as_tensor(np.asarray(want, dtype=np.float32))
+    want = want.to(got.device)
+    assert got.shape == want.shape, (what, tuple(got.shape), tuple(want.shape))
+    if got.numel() == 0:
+        return
+    tol = TOL[dtype]
+    bad = ~torch.isclose(got, want, **tol)
+    if bool(bad.any()):
+        idx = tuple(int(i) for i in bad.nonzero()[0])
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.numel()} elements outside rtol={tol['rtol']} atol={tol['atol']}; "
+                             f"first at {idx}: got {float(got[idx])} want {float(want[idx])}")
+    err = got - want
+    scale = float(want.abs().max())
+    worst = float(err.abs().max())
+    assert worst <= MAX_REL[dtype] * scale, f"{what}: max |got - want| = {worst:.3e} exceeds {MAX_REL[dtype]:.2e} x max |want| = {scale:.3e}"
+    rel = float(torch.linalg.vector_norm(err.double()) / torch.linalg.vector_norm(want.double()).clamp_min(1e-300))
+    assert rel <= RMS_REL[dtype], f"{what}: ||got - want|| / ||want|| = {rel:.3e} exceeds {RMS_REL[dtype]:.2e}"
 
 
 def assert_topology_equal(m, topo, what=""):

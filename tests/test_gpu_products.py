@@ -35,9 +35,18 @@ _GRID += [(*s, *t, 64, d) for s, t, d in itertools.product(_SMALL, _TRANSPOSE, _
 
 
 def _seed(*args):
-    s = abs(hash(tuple(str(a) for a in args))) % (2 ** 31)
+    """Seeds numpy and torch from the test's arguments; the same inputs in every process, so that a failure
+    seen once can be reproduced from its test id."""
+    s = U.stable_seed(*args)
     np.random.seed(s)
     torch.manual_seed(s)
+    return s
+
+
+def _incoming_gradient(shape, dtype):
+    """A seeded N(0, 1) gradient in the output's dtype: every block row and column of it is different, so a
+    backward pass that picked the wrong block of it, or its transpose inside a block, cannot pass."""
+    return torch.randn(*shape).to(dtype).to(DEV)
 
 
 def _dense(rows, cols, dtype, std=0.1):
@@ -64,15 +73,16 @@ def test_dsd(m, k, n, sparsity, trans_a, trans_b, blocking, dtype):
     want = O.dsd((m, k), U.np32(a.data), topo, trans_a, U.np32(rhs))
     U.assert_close(out, want, dtype, "dsd forward")
 
-    out.sum().backward()
-    ones = np.ones((m, n), dtype=np.float32)
+    g = _incoming_gradient((m, n), dtype)
+    out.backward(g)
+    g32 = U.np32(g)
     # d data: (dy rhs^T) sampled on the stored pattern (transposed when the operand is)
     rhs32 = U.np32(rhs)
-    want_data = O.sdd(rhs32, ones.T, topo) if trans_a else O.sdd(ones, rhs32.T, topo)
+    want_data = O.sdd(rhs32, g32.T, topo) if trans_a else O.sdd(g32, rhs32.T, topo)
     assert a.grad.data.shape == a.data.shape
     U.assert_close(a.grad.data, want_data, dtype, "dsd grad wrt sparse")
     # d rhs = op(S)^T dy, in the layout of b
-    want_rhs = O.dsd((k, m), U.np32(a.data), topo, not trans_a, ones)
+    want_rhs = O.dsd((k, m), U.np32(a.data), topo, not trans_a, g32)
     assert b.grad.shape == b.shape
     U.assert_close(b.grad, want_rhs.T if trans_b else want_rhs, dtype, "dsd grad wrt dense")
 
@@ -90,13 +100,14 @@ def test_dds(m, k, n, sparsity, trans_a, trans_b, blocking, dtype):
     want = O.dds(U.np32(lhs), (k, n), U.np32(b.data), topo, trans_b)
     U.assert_close(out, want, dtype, "dds forward")
 
-    out.sum().backward()
-    ones = np.ones((m, n), dtype=np.float32)
-    want_lhs = O.dds(ones, (n, k), U.np32(b.data), topo, not trans_b)
+    g = _incoming_gradient((m, n), dtype)
+    out.backward(g)
+    g32 = U.np32(g)
+    want_lhs = O.dds(g32, (n, k), U.np32(b.data), topo, not trans_b)
     assert a.grad.shape == a.shape
     U.assert_close(a.grad, want_lhs.T if trans_a else want_lhs, dtype, "dds grad wrt dense")
     lhs32 = U.np32(lhs)
-    want_data = O.sdd(ones.T, lhs32, topo) if trans_b else O.sdd(lhs32.T, ones, topo)
+    want_data = O.sdd(g32.T, lhs32, topo) if trans_b else O.sdd(lhs32.T, g32, topo)
     U.assert_close(b.grad.data, want_data, dtype, "dds grad wrt sparse")
 
 
@@ -116,10 +127,11 @@ def test_sdd(m, k, n, sparsity, trans_a, trans_b, blocking, dtype):
     # the reference's own comparator: dense product masked to the topology
     U.assert_close(out.data, O.dense_masked_sdd(U.np32(lhs), U.np32(rhs), topo), dtype, "sdd vs dense-masked")
 
-    stk.ops.sum(out).backward()
-    ones = np.ones(want.shape, dtype=np.float32)
-    want_lhs = O.dsd((m, n), ones, topo, False, U.np32(rhs).T)
-    want_rhs = O.dds(U.np32(lhs).T, (m, n), ones, topo, False)
+    g = _incoming_gradient(want.shape, dtype)
+    out.data.backward(g)
+    g32 = U.np32(g)
+    want_lhs = O.dsd((m, n), g32, topo, False, U.np32(rhs).T)
+    want_rhs = O.dds(U.np32(lhs).T, (m, n), g32, topo, False)
     U.assert_close(a.grad, want_lhs.T if trans_a else want_lhs, dtype, "sdd grad wrt lhs")
     U.assert_close(b.grad, want_rhs.T if trans_b else want_rhs, dtype, "sdd grad wrt rhs")
 
@@ -512,12 +524,12 @@ def _sliced_ran(fn):
     """Runs fn() with the dsd workspace cleared and reports whether the launch cut tiles into slices along k
     (it then wrote partial tiles into the workspace)."""
     from stk_amd.backend import hip_kernels
-    for ws in hip_kernels._dsd_workspaces.values():
+    for ws, _ in hip_kernels._dsd_workspaces.values():
         ws.zero_()
     out = fn()
     torch.cuda.synchronize()
     touched = False
-    for ws in hip_kernels._dsd_workspaces.values():
+    for ws, _ in hip_kernels._dsd_workspaces.values():
         touched = touched or bool(ws.count_nonzero().item() > 0)
     return out, touched
 
@@ -525,7 +537,7 @@ def _sliced_ran(fn):
 def _assert_counters_zero(m, n):
     from stk_amd.backend import hip_kernels
     counters = 4 * torch.cuda.get_device_properties(0).multi_processor_count
-    for ws in hip_kernels._dsd_workspaces.values():
+    for ws, _ in hip_kernels._dsd_workspaces.values():
         assert ws[:counters].count_nonzero().item() == 0, "counters of the sliced launch are not back at zero"
 
 
@@ -617,31 +629,189 @@ def test_dsd_sliced_last_round_random_pattern():
     assert y[3 * b:4 * b].count_nonzero().item() == 0 and y[25 * b:].count_nonzero().item() == 0
 
 
-def test_dmoe_config3_full_size_properties():
-    """16384 tokens, hidden 1024, ffn 4096, 64 experts, top-1: too big for the CPU
-    oracle in a test, so the full-size run is checked per expert against fp32
-    torch.matmul on the GPU (the block-diagonal structure makes every expert an
-    ordinary dense product) and through linearity."""
-    dtype = torch.bfloat16
-    tokens = U.dmoe_tokens_top1(16384, 64, 0)
-    topo, tm, x, w1, w2 = _dmoe_case(tokens, 1024, 4096, 128, dtype, 0)
-    pad = O.padded_tokens_per_expert(tokens, 128)
-    h = stk.ops.sdd(x, w1, tm)
-    y = stk.ops.dsd(h, w2)
-    dw1 = stk.ops.dds(x.t(), h)
-    w = 4096 // 128
+def _routed_topology(choices, blocking, ffn, dtype):
+    """Expert choices [tokens, top_k] -> (route result, topology Matrix with uninitialised values), both from the
+    library's own kernels (stk_route, stk_dmoe_topology), plus the padded rows per expert on the host."""
+    r = stk.ops.route(choices.to(DEV), 64, blocking)
+    rows = r.row_slots.numel()
+    tm = stk.ops.dmoe_topology(r.padded_bins, blocking, rows // blocking, ffn // blocking, dtype=dtype)
+    pad = np.diff(np.concatenate([[0], r.padded_bins.cpu().numpy()]))
+    return r, tm, pad
+
+
+def _expert_blocks(values, r0, p, ffn, b):
+    """The rows [r0, r0 + p) of a block-diagonal dMoE matrix (one expert) as a dense [p, ffn] tensor, gathered
+    from the blocked values [nnz, b, b] (ffn / b blocks per block row, block rows in order)."""
+    w, rb0, nb = ffn // b, r0 // b, p // b
+    return values[rb0 * w:(rb0 + nb) * w].reshape(nb, w, b, b).permute(0, 2, 1, 3).reshape(p, ffn)
+
+
+def _check_dmoe_products_full_size(choices, hidden, ffn, blocking, dtype, seed):
+    """The six products of a dMoE FFN, forward and backward, at full size on a routed topology.  Too big for the
+    CPU oracle inside a test; the block-diagonal structure makes every expert an ordinary dense product, so
+    each product is checked expert by expert against fp32 torch.matmul on the GPU on the same 16-bit inputs:
+    within the north-star tolerance and within the scale-free bounds of tests/_util.py.  The topology is
+    checked bit for bit against the oracle's closed form."""
+    r, tm, pad = _routed_topology(choices, blocking, ffn, dtype)
+    counts = np.bincount(choices.reshape(-1).numpy(), minlength=64)
+    assert np.array_equal(pad, O.padded_tokens_per_expert(counts, blocking))
+    U.assert_topology_equal(tm, O.dmoe_topology(counts, ffn, blocking), "routed topology")
+    rows, cols = tm.size()
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g, device=DEV) * 0.02).to(dtype)
+    x, w1, w2 = rnd(rows, hidden), rnd(hidden, cols), rnd(cols, hidden)
+    dy = rnd(rows, hidden)
+    h = stk.ops.sdd(x, w1, tm)                 # forward, layer 0
+    y = stk.ops.dsd(h, w2)                     # forward, layer 1
+    dw1 = stk.ops.dds(x.t(), h)                # weight gradient of layer 0 (h stands in for dh: same topology)
+    dw2 = stk.ops.dsd(h.t(), dy)               # weight gradient of layer 1
+    dx = stk.ops.dsd(h, w1.t())                # input gradient of layer 0
+    dh = stk.ops.sdd(dy, w2.t(), tm)           # gradient of the hidden activations
+    assert y.shape == (rows, hidden) and dw1.shape == (hidden, cols) and dw2.shape == (cols, hidden) and dx.shape == (rows, hidden)
     r0 = 0
-    for e, p in enumerate(pad):
+    for e, p in enumerate(int(v) for v in pad):
+        c0, c1 = e * ffn, (e + 1) * ffn
         if p == 0:
+            # an expert without tokens owns empty block columns: its weight gradients are exact zeros
+            assert dw1[:, c0:c1].count_nonzero().item() == 0 and dw2[c0:c1].count_nonzero().item() == 0, f"expert {e}"
             continue
-        xe = x[r0:r0 + p].float()
-        he = xe @ w1[:, e * 4096:(e + 1) * 4096].float()
-        rb0, nb = r0 // 128, p // 128
-        got = h.data[rb0 * w:(rb0 + nb) * w].reshape(nb, w, 128, 128).permute(0, 2, 1, 3).reshape(p, 4096)
-        U.assert_close(got, he.cpu().numpy(), dtype, f"expert {e} sdd")
-        hb = got.float()
-        U.assert_close(y[r0:r0 + p], (hb @ w2[e * 4096:(e + 1) * 4096].float()).cpu().numpy(), dtype, f"expert {e} dsd")
-        U.assert_close(dw1[:, e * 4096:(e + 1) * 4096], (xe.t() @ hb).cpu().numpy(), dtype, f"expert {e} dds")
+        xe, dye = x[r0:r0 + p].float(), dy[r0:r0 + p].float()
+        w1e, w2e = w1[:, c0:c1].float(), w2[c0:c1].float()
+        he = _expert_blocks(h.data, r0, p, ffn, blocking)
+        U.assert_close_scaled(he, xe @ w1e, dtype, f"expert {e} sdd(x, W1)")
+        hf = he.float()
+        U.assert_close_scaled(y[r0:r0 + p], hf @ w2e, dtype, f"expert {e} dsd(h, W2)")
+        U.assert_close_scaled(dw1[:, c0:c1], xe.t() @ hf, dtype, f"expert {e} dds(x^T, h)")
+        U.assert_close_scaled(dw2[c0:c1], hf.t() @ dye, dtype, f"expert {e} dsd(h^T, dy)")
+        U.assert_close_scaled(dx[r0:r0 + p], hf @ w1e.t(), dtype, f"expert {e} dsd(h, W1^T)")
+        U.assert_close_scaled(_expert_blocks(dh.data, r0, p, ffn, blocking), dye @ w2e.t(), dtype, f"expert {e} sdd(dy, W2^T)")
         r0 += p
-    # linearity in the dense operand: dsd(h, 2 w2) == 2 dsd(h, w2) exactly (power-of-two scaling)
-    assert torch.equal(stk.ops.dsd(h, w2 * 2), y * 2)
+    assert r0 == rows
+    # linearity in the dense operand: dsd(h, 2 w2) == 2 dsd(h, w2) exactly (power-of-two scaling), wherever the
+    # sum is a normal number of the 16-bit type (float16 rounds sums below 2^-14 on a fixed grid; a rounded value of
+    # at least 2^-13 cannot come from such a sum)
+    y2 = stk.ops.dsd(h, w2 * 2)
+    normal = y.float().abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y * 2)[normal]) and float(normal.float().mean()) > 0.9
+
+
+def _top1_choices(tokens, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(tokens, 64, generator=g).argmax(dim=1, keepdim=True).to(torch.int32)
+
+
+def test_dmoe_config3_full_size():
+    # 16384 tokens, top-1 over 64 experts from N(0, 1) logits, hidden 1024, ffn 4096, blocking 128, bf16
+    _check_dmoe_products_full_size(_top1_choices(16384, 0), 1024, 4096, 128, torch.bfloat16, 3)
+
+
+def test_dmoe_config4_full_size():
+    # 32768 tokens, top-2 from Zipf(1.2)-skewed popularity (Gumbel trick), hidden 2048, ffn 8192, blocking 128, bf16
+    g = torch.Generator().manual_seed(0)
+    logp = -1.2 * torch.log(torch.arange(1, 65, dtype=torch.float64))
+    u = torch.rand(32768, 64, generator=g, dtype=torch.float64).clamp_min(1e-300)
+    choices = (logp[None, :] - torch.log(-torch.log(u))).topk(2, dim=1).indices.to(torch.int32)
+    _check_dmoe_products_full_size(choices, 2048, 8192, 128, torch.bfloat16, 4)
+
+
+def test_dmoe_config5_full_size():
+    # config 3's routing with blocking 64 and fp16
+    _check_dmoe_products_full_size(_top1_choices(16384, 0), 1024, 4096, 64, torch.float16, 5)
+
+
+def test_dmoe_config5_extreme_skew_full_size():
+    # one expert takes half of the 16384 tokens, the others share the rest; blocking 64, fp16
+    g = torch.Generator().manual_seed(0)
+    top = torch.randint(1, 64, (16384,), generator=g, dtype=torch.int32)
+    top[torch.randperm(16384, generator=g)[:8192]] = 0
+    _check_dmoe_products_full_size(top[:, None], 1024, 4096, 64, torch.float16, 6)
+
+
+@pytest.mark.parametrize("dtype", _DTYPES)
+def test_config1_seed0_mask_all_products(dtype):
+    """BASELINE configuration 1 on the HIP path: stk.random.mask(1024, 1024, 0.5, 128) from numpy seed 0 (the
+    known-answer topology of tests/golden/config1_topology.json), dense operands 1024 x 1024 ~ N(0, 1) from torch
+    seed 0 rounded to the 16-bit type the kernels compute in, sdd / dsd / dds in all four transpose variants
+    against the oracle.  (The reference runs this configuration in fp32 on the host; the products here take
+    float16 / bfloat16 device tensors only.)  With N(0, 1) operands the sums are ~32, far above the absolute
+    tolerance, so the comparison is a relative one."""
+    import json
+    import os
+    np.random.seed(0)
+    torch.manual_seed(0)
+    s = stk.random.mask(1024, 1024, 0.5, 128)
+    with open(os.path.join(os.path.dirname(__file__), "golden", "config1_topology.json")) as f:
+        golden = json.load(f)
+    for name in ("row_indices", "column_indices", "offsets", "offsets_t", "column_indices_t", "block_offsets_t"):
+        assert getattr(s, name).tolist() == golden[name], name
+    values = torch.randn(s.data.shape).to(dtype)
+    s = stk.Matrix(s.size(), values, s.row_indices, s.column_indices, s.offsets, s.column_indices_t, s.offsets_t, s.block_offsets_t).to(DEV)
+    a = torch.randn(1024, 1024).to(dtype).to(DEV)
+    b = torch.randn(1024, 1024).to(dtype).to(DEV)
+    topo = U.topo_of(s)
+    data32, a32, b32 = U.np32(s.data), U.np32(a), U.np32(b)
+    for ta, tb in _TRANSPOSE:
+        lhs, lhs32 = (a.t(), a32.T) if ta else (a, a32)
+        rhs, rhs32 = (b.t(), b32.T) if tb else (b, b32)
+        U.assert_close_scaled(stk.ops.sdd(lhs, rhs, s).data, O.sdd(lhs32, rhs32, topo), dtype, f"sdd {ta} {tb}")
+        U.assert_close_scaled(stk.ops.dsd(s.t() if ta else s, rhs), O.dsd((1024, 1024), data32, topo, ta, rhs32), dtype, f"dsd {ta} {tb}")
+        U.assert_close_scaled(stk.ops.dds(lhs, s.t() if tb else s), O.dds(lhs32, (1024, 1024), data32, topo, tb), dtype, f"dds {ta} {tb}")
+    # the reference's own comparator for this configuration: to_dense + matmul, masked to the topology
+    dense = stk.ops.to_dense(s).float()
+    U.assert_close_scaled(stk.ops.dsd(s, b), dense @ b.float(), dtype, "dsd vs to_dense + matmul")
+    U.assert_close_scaled(stk.ops.dds(a, s), a.float() @ dense, dtype, "dds vs to_dense + matmul")
+    U.assert_close_scaled(stk.ops.sdd(a, b, s).data, O.dense_masked_sdd(a32, b32, topo), dtype, "sdd vs matmul masked to the topology")
+
+
+def test_products_on_a_topology_built_in_inference_mode():
+    # tensors made under inference mode keep no version counter; the fusion plan must not need one
+    dtype = torch.bfloat16
+    _seed("inference")
+    with torch.inference_mode():
+        choices = torch.randint(0, 64, (4096, 1), dtype=torch.int32)
+        r = stk.ops.route(choices.to(DEV), 64, 128)
+        tm = stk.ops.dmoe_topology(r.padded_bins, 128, r.row_slots.numel() // 128, 4, dtype=dtype)
+        assert tm.offsets.is_inference()
+        rows, cols = tm.size()
+        x, w1, w2 = ((torch.randn(*shape) * 0.05).to(dtype).to(DEV) for shape in ((rows, 256), (256, cols), (cols, 256)))
+        h = stk.ops.sdd(x, w1, tm)
+        y = stk.ops.dsd(h, w2)
+        dw1 = stk.ops.dds(x.t(), h)
+        s = stk.ops.to_sparse(stk.ops.to_dense(h), 128)
+        assert torch.equal(s.data, h.data)
+    topo = U.topo_of(tm)
+    U.assert_close(h.data, O.sdd(U.np32(x), U.np32(w1), topo), dtype, "sdd in inference mode")
+    U.assert_close(y, O.dsd(topo.shape, U.np32(h.data), topo, False, U.np32(w2)), dtype, "dsd in inference mode")
+    U.assert_close(dw1, O.dds(U.np32(x).T, topo.shape, U.np32(h.data), topo, False), dtype, "dds in inference mode")
+
+
+def test_fusion_plan_follows_replaced_column_indices():
+    # one offsets tensor (a fixed number of blocks per row) used with column indices that are replaced by a new
+    # tensor of the same size: the caching allocator hands the new one the old address, and a plan kept for the
+    # old pattern (rows marked identical) would compute the wrong blocks
+    from stk_amd.backend import hip_kernels
+    dtype = torch.bfloat16
+    _seed("replaced indices")
+    b, rb, cb, per_row = 128, 24, 16, 4
+    offsets = (torch.arange(rb + 1, dtype=torch.int32) * per_row).to(DEV)
+    x = _dense(rb * b, 256, dtype, 0.05).detach()
+    w = _dense(256, cb * b, dtype, 0.05).detach()
+    v = _dense(cb * b, 256, dtype, 0.05).detach()
+    for trial, identical_rows in enumerate((True, False, True, False)):
+        if identical_rows:
+            cols = np.tile(np.arange(per_row) * 3, (rb, 1))
+        else:
+            cols = np.stack([np.sort(np.random.choice(cb, per_row, replace=False)) for _ in range(rb)])
+        ci = torch.from_numpy(cols.reshape(-1).astype(np.int16)).to(DEV)
+        ri = torch.arange(rb, dtype=torch.int16).repeat_interleave(per_row).to(DEV)
+        data = torch.empty(rb * per_row, b, b, dtype=dtype, device=DEV)
+        m = stk.Matrix(torch.Size((rb * b, cb * b)), data, ri, ci, offsets)
+        topo = U.topo_of(m)
+        out = stk.ops.sdd(x, w, m)
+        U.assert_close(out.data, O.sdd(U.np32(x), U.np32(w), topo), dtype, f"sdd, trial {trial}")
+        U.assert_close(stk.ops.dsd(out, v), O.dsd(topo.shape, U.np32(out.data), topo, False, U.np32(v)), dtype, f"dsd, trial {trial}")
+        U.assert_close(stk.ops.dds(x.t(), out), O.dds(U.np32(x).T, topo.shape, U.np32(out.data), topo, False), dtype, f"dds, trial {trial}")
+        cached = offsets._stk_plan
+        assert cached[0][0] is ci          # the entry holds the tensors it describes
+        del m, ci, out, topo               # only the cache keeps the old column indices alive now
+    assert hip_kernels.fusion_plan(offsets, cached[0][0], blocking=128) is cached[1]

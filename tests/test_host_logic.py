@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().stk_abi_version() == 8
+    assert _lib.load().stk_abi_version() == _lib.ABI_VERSION
     assert _lib.load().stk_transpose_meta_workspace_bytes(1000) >= 4 * 4 * 1000
 
 
@@ -196,3 +196,39 @@ def test_bench_rejects_what_it_does_not_measure():
         run = subprocess.run([sys.executable, os.path.join(root, "bench.py")] + flags, capture_output=True, text=True, timeout=300)
         assert run.returncode != 0
         assert text in run.stderr, run.stderr
+
+
+def test_fusion_plan_cache_is_tied_to_the_index_tensors_it_was_built_from():
+    # the plan of a topology is cached on its offsets tensor; the entry holds the other index tensors, so that
+    # a new tensor at a recycled address, an in-place change or a tensor without a version counter miss
+    from stk_amd.backend import hip_kernels as hk
+    offsets = torch.arange(0, 20, 4, dtype=torch.int32)
+    ci = torch.tensor([0, 1, 2, 3] * 4, dtype=torch.int16)
+    ot, cit = torch.arange(0, 20, 4, dtype=torch.int32), torch.tensor([0, 1, 2, 3] * 4, dtype=torch.int16)
+    plan = object()
+    assert hk._plan_cache_get((offsets, ci), 128) is None
+    assert hk._plan_cache_put((offsets, ci, ot, cit), 128, plan, 7, None)
+    assert hk._plan_cache_get((offsets, ci, ot, cit), 128)[1] is plan
+    assert hk._plan_cache_get((offsets, ci), 128)[1] is plan               # a request without the transpose metadata
+    assert hk._plan_cache_get((offsets, ci, ot, cit), 64) is None          # another blocking
+    # the column indices replaced by an equal-sized tensor: a miss, and the old tensor is still alive in the entry
+    held = offsets._stk_plan[0][0]
+    assert held is ci
+    address = ci.data_ptr()
+    del ci
+    other = torch.tensor([3, 2, 1, 0] * 4, dtype=torch.int16)
+    assert held.data_ptr() == address and other.data_ptr() != address
+    assert hk._plan_cache_get((offsets, other, ot, cit), 128) is None
+    # modified in place: the version counter moves
+    assert hk._plan_cache_get((offsets, held, ot, cit), 128)[1] is plan
+    held[0] = 5
+    assert hk._plan_cache_get((offsets, held, ot, cit), 128) is None
+    # a plan built without the transpose metadata does not serve a request with it
+    assert hk._plan_cache_put((offsets, held), 128, plan, 7, None)
+    assert hk._plan_cache_get((offsets, held, ot, cit), 128) is None
+    # tensors made under inference mode keep no version counter: never cached, and asking does not raise
+    with torch.inference_mode():
+        frozen = torch.arange(0, 20, 4, dtype=torch.int32)
+        fci = torch.zeros(16, dtype=torch.int16)
+    assert not hk._plan_cache_put((frozen, fci), 128, plan, 7, None)
+    assert hk._plan_cache_get((frozen, fci), 128) is None
