@@ -303,6 +303,23 @@ int stk_route(const int32_t* top_experts, int64_t slots, int64_t num_experts, in
               void* workspace, size_t workspace_bytes, stk_stream_t stream);
 
 /*
+ * stk_route for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same three launches with the same
+ * outputs, bit for bit, but the per-tile table lives in a device array that belongs to the library
+ * (STK_ROUTE_STATIC_MAX_ENTRIES int32 entries = 4 MiB on every GPU the library runs on, held until the process
+ * ends).  No counterpart in the reference.  The call allocates nothing and frees nothing; the first call on a
+ * device resolves the array's address on that device (make it outside a capture).  Sizes with
+ * num_experts * ceil(slots / 256) > STK_ROUTE_STATIC_MAX_ENTRIES are refused with STK_ERR_WORKSPACE.  All calls
+ * on one GPU share the array: calls that may overlap on one GPU (different streams without an ordering between
+ * them) race; calls on one stream, or ordered by events, do not.  The table needs no clearing between calls
+ * (every entry that is read is written first).
+ */
+#define STK_ROUTE_STATIC_MAX_ENTRIES (1 << 20)
+int stk_route_static(const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
+                     int32_t* indices, int32_t* bin_ids, int32_t* bins, int32_t* padded_bins,
+                     int32_t* slot_rows, int32_t* row_slots, stk_stream_t stream);
+
+/*
  * Rows of x [tokens, cols] copied into the padded layout: out[r] = x[row_slots[r] / top_k],
  * zeros where row_slots[r] < 0.  With weights (fp32, one per slot, or NULL) the row is
  * multiplied by weights[row_slots[r]] in fp32 and rounded once (this is the gradient of

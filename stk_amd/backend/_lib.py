@@ -41,6 +41,7 @@ SIGNATURES = {
     "stk_dmoe_topology": (_int, [_p, _i64, _int, _i64, _i64, _int, _p, _p, _p, _p, _p, _p, _p]),
     "stk_route_workspace_bytes": (_sz, [_i64, _i64]),
     "stk_route": (_int, [_p, _i64, _i64, _int, _i64, _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "stk_route_static": (_int, [_p, _i64, _i64, _int, _i64, _p, _p, _p, _p, _p, _p, _p]),
     "stk_padded_gather": (_int, [_p, _i64, _i64, _i64, _p, _p, _int, _i64, _p, _i64, _int, _p]),
     "stk_padded_scatter": (_int, [_p, _i64, _i64, _i64, _p, _p, _int, _i64, _p, _i64, _int, _p]),
     "stk_padded_scatter_weight_gradient": (_int, [_p, _i64, _i64, _i64, _p, _i64, _p, _int, _i64, _p, _int, _p]),

@@ -3,6 +3,8 @@
 // counting sort and lays every expert's rows out in a bin padded to the block size;
 // stk_padded_gather / stk_padded_scatter move the token rows into that layout and back.
 // The index work is bit-exact by construction; the copies move 16 bytes per lane.
+#include <atomic>
+
 #include "common.h"
 #include "wave_scan.h"
 
@@ -363,23 +365,29 @@ extern "C" size_t stk_route_workspace_bytes(int64_t slots, int64_t num_experts) 
   return static_cast<size_t>(num_experts * (tiles > 0 ? tiles : 1)) * sizeof(int32_t);
 }
 
-extern "C" int stk_route(const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
-                         int32_t* indices, int32_t* bin_ids, int32_t* bins, int32_t* padded_bins,
-                         int32_t* slot_rows, int32_t* row_slots, void* workspace, size_t workspace_bytes, stk_stream_t stream) {
+// Argument checks shared by the two routing entry points.
+static int route_check(const char* who, const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
+                       const int32_t* indices, const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins,
+                       const int32_t* slot_rows, const int32_t* row_slots) {
   if (slots < 0 || num_experts <= 0 || blocking <= 0 || padded_rows < 0)
-    return fail(STK_ERR_DIMS, "stk_route: %lld slots, %lld experts, blocking %d, %lld rows", (long long)slots, (long long)num_experts,
+    return fail(STK_ERR_DIMS, "%s: %lld slots, %lld experts, blocking %d, %lld rows", who, (long long)slots, (long long)num_experts,
                 blocking, (long long)padded_rows);
-  if (num_experts > kMaxExperts) return fail(STK_ERR_UNSUPPORTED, "stk_route: at most %d experts", kMaxExperts);
+  if (num_experts > kMaxExperts) return fail(STK_ERR_UNSUPPORTED, "%s: at most %d experts", who, kMaxExperts);
   if (slots + num_experts * (int64_t)blocking > INT32_MAX || padded_rows > INT32_MAX)
-    return fail(STK_ERR_UNSUPPORTED, "stk_route: size exceeds 32-bit range");
+    return fail(STK_ERR_UNSUPPORTED, "%s: size exceeds 32-bit range", who);
   if (!bins || !padded_bins || (slots > 0 && (!top_experts || !indices || !bin_ids || !slot_rows)) || (padded_rows > 0 && !row_slots))
-    return fail(STK_ERR_DIMS, "stk_route: missing pointer");
-  if (!workspace || workspace_bytes < stk_route_workspace_bytes(slots, num_experts))
-    return fail(STK_ERR_WORKSPACE, "stk_route: workspace of %zu bytes needed", stk_route_workspace_bytes(slots, num_experts));
-  hipStream_t s = static_cast<hipStream_t>(stream);
+    return fail(STK_ERR_DIMS, "%s: missing pointer", who);
+  return STK_OK;
+}
+
+// The three launches of a routing; `table` holds stk_route_workspace_bytes(slots, num_experts) bytes.  Every entry of
+// the table that is read is written first (the histogram writes a count for every expert of every tile), so the
+// table needs no initial value.
+static void route_launch(const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
+                         int32_t* indices, int32_t* bin_ids, int32_t* bins, int32_t* padded_bins, int32_t* slot_rows, int32_t* row_slots,
+                         int32_t* table, hipStream_t s) {
   const int real_tiles = (int)((slots + kRouteTile - 1) / kRouteTile);
   const int tiles = real_tiles > 0 ? real_tiles : 1;   // one tile without slots still clears its counts and row_slots
-  int32_t* table = static_cast<int32_t*>(workspace);
   int bits = 0;
   while (((int64_t)1 << bits) < num_experts) bits++;
   hipLaunchKernelGGL(route_histogram_kernel, dim3(tiles), dim3(kWave), 0, s, top_experts, slots, (int)num_experts, tiles, table,
@@ -388,7 +396,68 @@ extern "C" int stk_route(const int32_t* top_experts, int64_t slots, int64_t num_
   if (slots > 0)
     hipLaunchKernelGGL(route_scatter_kernel, dim3(tiles), dim3(kWave), 0, s, top_experts, slots, (int)num_experts, bits, tiles, table,
                        bins, padded_bins, indices, bin_ids, slot_rows, row_slots, padded_rows);
+}
+
+extern "C" int stk_route(const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
+                         int32_t* indices, int32_t* bin_ids, int32_t* bins, int32_t* padded_bins,
+                         int32_t* slot_rows, int32_t* row_slots, void* workspace, size_t workspace_bytes, stk_stream_t stream) {
+  const int rc = route_check("stk_route", top_experts, slots, num_experts, blocking, padded_rows, indices, bin_ids, bins, padded_bins,
+                             slot_rows, row_slots);
+  if (rc != STK_OK) return rc;
+  if (!workspace || workspace_bytes < stk_route_workspace_bytes(slots, num_experts))
+    return fail(STK_ERR_WORKSPACE, "stk_route: workspace of %zu bytes needed", stk_route_workspace_bytes(slots, num_experts));
+  route_launch(top_experts, slots, num_experts, blocking, padded_rows, indices, bin_ids, bins, padded_bins, slot_rows, row_slots,
+               static_cast<int32_t*>(workspace), static_cast<hipStream_t>(stream));
   return check_launch("stk_route");
+}
+
+// ---------------------------------------------------------------- routing without a workspace argument
+// The table of stk_route kept in device memory that belongs to the library: one array per GPU, there from the moment
+// the code object is loaded until the process ends.  Host code never uses the array's name as an address: its
+// address on a device is asked for once, with that device current, and kept.
+namespace stk {
+constexpr size_t kRouteScratchBytes = STK_ROUTE_STATIC_MAX_ENTRIES * sizeof(int32_t);
+static __device__ __align__(256) unsigned char route_scratch[kRouteScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> route_scratch_of_device[kMaxDevices];
+
+// Address of route_scratch on the current device (null with the error set when it cannot be had).
+static void* route_scratch_address() {
+  int dev = -1;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(STK_ERR_HIP, "stk_route_static: no usable current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "device index out of range");
+    return nullptr;
+  }
+  void* p = route_scratch_of_device[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  const hipError_t r = hipGetSymbolAddress(&p, HIP_SYMBOL(route_scratch));
+  if (r != hipSuccess || !p) {
+    fail(STK_ERR_HIP, "stk_route_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(r));
+    return nullptr;
+  }
+  route_scratch_of_device[dev].store(p, std::memory_order_release);   // every thread that asks gets the same answer
+  return p;
+}
+}  // namespace stk
+
+extern "C" int stk_route_static(const int32_t* top_experts, int64_t slots, int64_t num_experts, int blocking, int64_t padded_rows,
+                                int32_t* indices, int32_t* bin_ids, int32_t* bins, int32_t* padded_bins,
+                                int32_t* slot_rows, int32_t* row_slots, stk_stream_t stream) {
+  const int rc = route_check("stk_route_static", top_experts, slots, num_experts, blocking, padded_rows, indices, bin_ids, bins,
+                             padded_bins, slot_rows, row_slots);
+  if (rc != STK_OK) return rc;
+  const size_t need = stk_route_workspace_bytes(slots, num_experts);
+  if (need > kRouteScratchBytes)
+    return fail(STK_ERR_WORKSPACE,
+                "stk_route_static: %lld slots over %lld experts need a table of %zu bytes, the built-in one holds %zu "
+                "(experts x ceil(slots / %d) <= %d); use stk_route with a workspace",
+                (long long)slots, (long long)num_experts, need, kRouteScratchBytes, kRouteTile, STK_ROUTE_STATIC_MAX_ENTRIES);
+  void* table = route_scratch_address();
+  if (!table) return STK_ERR_HIP;
+  route_launch(top_experts, slots, num_experts, blocking, padded_rows, indices, bin_ids, bins, padded_bins, slot_rows, row_slots,
+               static_cast<int32_t*>(table), static_cast<hipStream_t>(stream));
+  return check_launch("stk_route_static");
 }
 
 extern "C" int stk_padded_gather(const void* x, int64_t tokens, int64_t cols, int64_t x_stride, const int32_t* row_slots,
