@@ -10,18 +10,29 @@ the block-diagonal topology [T', 64 * 4096] with 128 x 128 blocks.  One step is
 and the metric is effective TFLOP/s over nonzero blocks, nnz * 2 * 128^2 * 1024
 FLOP per product.  Inputs are synthetic and resident in HBM before timing.
 
+Order of the run: the same-problem dense GEMMs and the routing are timed first (they also bring
+the GPU to its steady clocks: the first ~100 ms of work after an idle period run up to 15 % slower),
+then W untimed steps, then K steps timed by the wall clock between two synchronisations with nothing
+but the three launches inside (`value`, `ms_per_step`), then K more steps with a HIP event between the
+launches (`per_op_ms`, `roofline`), then each product K times back to back between one pair of events
+(`per_op_back_to_back_ms`).
+
 The JSON line also carries
   dense      same-problem dense bf16 GEMMs (torch.bmm over experts with the same
              FLOPs and weight bytes) timed in the same run, and our fraction of them
   roofline   algorithmic bytes (or FLOPs) of the slowest of the three kernels over
-             its mean duration from HIP events on the launch stream
+             its mean duration from HIP events on the launch stream; `traffic` is read
+             from the rocprofv3 counter summary under profiles/ (its source is named)
   routing    the token routing on either side of the products on the same workload
              (sort into padded expert bins, gather, scatter), timed outside the step
-  other_configs  (--configs 2,4,5,5skew) per-product times on the other configurations
-  cpu_baseline  the CPU oracle (block-walk port of the reference kernels) timed
-             on the host cores on a bounded sample of the same workload
+  other_configs  per-product times on the other configurations of BASELINE.json with their
+             dense comparators (--configs none leaves them out)
+  cpu_baseline  the reference's dense-equivalent CPU path (to_dense + torch.matmul + mask, fp32)
+             restated on the oracle's format helpers and timed on the host cores on a bounded,
+             scaled-down sample of the same workload; the oracle's block walk beside it
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -82,6 +93,18 @@ def time_events(fn, steps, warmup):
     return float(np.median([s.elapsed_time(e) for s, e in ev]))
 
 
+def time_batch(fn, calls):
+    """Mean time of `calls` launches issued back to back between one pair of events."""
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(calls):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / calls
+
+
 def dense_comparators(rows, dev, steps, warmup):
     """Same-problem dense GEMMs: every expert gets rows/EXPERTS token rows, so FLOPs
     and weight bytes equal the block-sparse products'."""
@@ -92,10 +115,10 @@ def dense_comparators(rows, dev, steps, warmup):
     he = torch.bmm(xe, w1)
     flops = 2.0 * EXPERTS * te * HIDDEN * FFN
     out = {"tokens_per_expert": te}
-    out["sdd_like_ms"] = time_events(lambda: torch.bmm(xe, w1), steps, warmup)
-    out["dsd_like_ms"] = time_events(lambda: torch.bmm(he, w2), steps, warmup)
-    out["dds_like_ms"] = time_events(lambda: torch.bmm(xe.transpose(1, 2), he), steps, warmup)
-    for k in ("sdd", "dsd", "dds"):
+    fns = {"sdd": lambda: torch.bmm(xe, w1), "dsd": lambda: torch.bmm(he, w2), "dds": lambda: torch.bmm(xe.transpose(1, 2), he)}
+    for k, fn in fns.items():
+        out[k + "_like_ms"] = time_events(fn, steps, warmup)              # one pair of events per call, median
+        out[k + "_like_back_to_back_ms"] = time_batch(fn, steps)          # one pair of events around `steps` calls
         out[k + "_like_tflops"] = flops / (out[k + "_like_ms"] * 1e-3) / 1e12
     # one plain GEMM with the same FLOPs (reads 1/64 of the weights): upper bound
     xa = (torch.randn(EXPERTS * te, HIDDEN, device=dev) * 0.02).bfloat16()
@@ -105,26 +128,31 @@ def dense_comparators(rows, dev, steps, warmup):
     return out
 
 
-def cpu_baseline(tokens_per_expert, budget_s=12.0):
-    """Times the CPU oracle (numpy port of the reference kernels' block walk) on
-    the experts of the same workload, cycling over them until the time budget is used."""
-    from oracle import stk_oracle as O
+def _blas_threads():
     try:
         from threadpoolctl import threadpool_info
-        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+        return int(max([p.get("num_threads", 1) for p in threadpool_info()] or [1]))
     except Exception:
-        threads = os.cpu_count() or 1
+        return os.cpu_count() or 1
+
+
+def cpu_block_walk(tokens_per_expert, budget_s):
+    """The CPU oracle's block walk (numpy port of the reference kernels) on the experts of the same workload,
+    one expert at a time, cycling over them until the time budget is used."""
+    from oracle import stk_oracle as O
     rng = np.random.RandomState(0)
+    max_rows = int(max((int(t) + BLOCK - 1) // BLOCK * BLOCK for t in tokens_per_expert))
+    # operands drawn once (outside the timed part); every expert takes its rows of x
+    x_all = rng.randn(max_rows, HIDDEN).astype(np.float32) * 0.02
+    w1 = rng.randn(HIDDEN, FFN).astype(np.float32) * 0.02
+    w2 = rng.randn(FFN, HIDDEN).astype(np.float32) * 0.02
     done_flops, elapsed, used = 0.0, 0.0, 0
     while elapsed < budget_s:
         for e, t in enumerate(tokens_per_expert):
             if t == 0:
                 continue
             topo = O.dmoe_topology([t], FFN, BLOCK)
-            rows = topo.shape[0]
-            x = rng.randn(rows, HIDDEN).astype(np.float32) * 0.02
-            w1 = rng.randn(HIDDEN, FFN).astype(np.float32) * 0.02
-            w2 = rng.randn(FFN, HIDDEN).astype(np.float32) * 0.02
+            x = x_all[:topo.shape[0]]
             t0 = time.perf_counter()
             h = O.sdd(x, w1, topo)
             O.dsd(topo.shape, h, topo, False, w2)
@@ -134,9 +162,57 @@ def cpu_baseline(tokens_per_expert, budget_s=12.0):
             used += 1
             if elapsed >= budget_s:
                 break
-    return {"value": done_flops / elapsed / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+    return {"value": done_flops / elapsed / 1e12, "unit": "TFLOP/s", "cores": _blas_threads(),
             "sample": f"oracle sdd+dsd+dds (fp32 numpy block walk, one expert at a time) over {used} expert problems of the same "
                       f"topology ({used / EXPERTS:.1f} passes over the {EXPERTS} experts), {elapsed:.1f} s of CPU work"}
+
+
+def cpu_baseline(tokens_per_expert, budget_s=8.0, group=4):
+    """The reference's dense-equivalent path on the host cores: to_dense(S), torch.matmul in fp32, and the
+    result masked to the topology (what stk's own tests compare its kernels with).  The whole topology as a
+    dense matrix would hold 20096 x 262144 values, so the experts are taken `group` at a time: each problem is
+    the block-diagonal topology of `group` consecutive experts with their real token counts, and the dense
+    product does `group` times the nonzero FLOPs (the full topology would do 64 times).  Throughput is counted
+    over the nonzero blocks only, as for the GPU.  The format helpers are the oracle's."""
+    from oracle import stk_oracle as O
+    g = torch.Generator().manual_seed(0)
+    threads = torch.get_num_threads()
+    cols = group * FFN
+    max_rows = int(max(sum((int(t) + BLOCK - 1) // BLOCK * BLOCK for t in tokens_per_expert[e0:e0 + group]) for e0 in range(0, EXPERTS, group)))
+    # operands drawn once (outside the timed part); every problem takes its rows of x
+    x_all = torch.randn(max_rows, HIDDEN, generator=g) * 0.02
+    w1 = torch.randn(HIDDEN, cols, generator=g) * 0.02
+    w2 = torch.randn(cols, HIDDEN, generator=g) * 0.02
+    done_flops, elapsed, problems = 0.0, 0.0, 0
+    while elapsed < budget_s:
+        for e0 in range(0, EXPERTS, group):
+            counts = [int(t) for t in tokens_per_expert[e0:e0 + group]]
+            if sum(counts) == 0:
+                continue
+            topo = O.dmoe_topology(counts, FFN, BLOCK)
+            rows = topo.shape[0]
+            x = x_all[:rows]
+            blocks = torch.zeros(rows // BLOCK, cols // BLOCK)
+            blocks[torch.from_numpy(topo.row_indices.astype(np.int64)), torch.from_numpy(topo.column_indices.astype(np.int64))] = 1.0
+            mask = blocks.repeat_interleave(BLOCK, 0).repeat_interleave(BLOCK, 1)     # to_dense of a matrix of ones
+            t0 = time.perf_counter()
+            h_dense = torch.matmul(x, w1) * mask                             # sdd: dense product, masked to the topology
+            y = torch.matmul(h_dense, w2)                                    # dsd: to_dense(h) @ W2
+            dw1 = torch.matmul(x.t(), h_dense)                               # dds: x^T @ to_dense(h)
+            elapsed += time.perf_counter() - t0
+            del y, dw1
+            done_flops += 3 * len(topo.row_indices) * 2.0 * BLOCK * BLOCK * HIDDEN
+            problems += 1
+            if elapsed >= budget_s:
+                break
+    out = {"value": done_flops / elapsed / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+           "host_cpu_count": os.cpu_count(), "torch_num_threads": int(threads),
+           "sample": f"dense-equivalent sdd+dsd+dds (torch.matmul fp32 on dense operands, sdd masked to the topology) over {problems} "
+                     f"problems of {group} consecutive experts of the same topology with their real token counts (1/{EXPERTS // group} "
+                     f"of the experts each, so the dense products do {group}x the nonzero FLOPs; the full topology would do "
+                     f"{EXPERTS}x), {elapsed:.1f} s of CPU work; TFLOP/s counted over nonzero blocks"}
+    out["block_walk"] = cpu_block_walk(tokens_per_expert, budget_s)
+    return out
 
 
 def routing_times(dev, steps, warmup, seed=0):
@@ -292,13 +368,24 @@ def other_config(name, dev, steps, warmup):
     return out
 
 
-# HBM bytes per launch on this workload from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the
-# scales a plain 1 GiB -> 1 GiB elementwise kernel gives); summary in profiles/bench_dmoe_fwd_hbm_counters.txt.
-MEASURED_HBM_BYTES = {"sdd_fused_kernel": 777.7e6, "dsd_sliced_kernel": 864.3e6, "dds_fused_kernel": 743.2e6}
+# HBM bytes per launch on this workload come from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, scaled by what the
+# same counters read for a plain copy of known size); the tracked summary of that run is read here, so that the
+# figure in the JSON line is the one in the repository and names its source.
+HBM_COUNTER_SUMMARY = os.path.join("profiles", "bench_dmoe_fwd_hbm_counters.txt")
 
 
 def measured_hbm_traffic(kernel):
-    return MEASURED_HBM_BYTES.get(kernel)
+    """(bytes per launch, source) for `kernel` from the 'total MB' column of the counter summary, or (None, reason)."""
+    path = os.path.join(ROOT, HBM_COUNTER_SUMMARY)
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) >= 8 and parts[0] == kernel:
+                    return float(parts[5]) * 1e6, HBM_COUNTER_SUMMARY
+    except OSError as err:
+        return None, f"{HBM_COUNTER_SUMMARY}: {err.strerror}"
+    return None, f"{HBM_COUNTER_SUMMARY}: no line for {kernel}"
 
 
 def main():
@@ -306,18 +393,21 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--preheat-ms", type=float, default=150.0,
+                    help="milliseconds of untimed steps before the W warm-up steps: after an idle period the GPU takes about "
+                         "40 ms of continuous work to reach its steady clocks (the first steps run up to 25 %% slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB -> 1 GiB elementwise kernel (torch.neg), the known-size reference for the HBM counters")
-    ap.add_argument("--configs", default="",
-                    help="comma-separated other configurations of BASELINE.json to time as well (2, 4, 5, 5skew); off by default")
+    ap.add_argument("--configs", default="2,4,5,5skew",
+                    help="comma-separated other configurations of BASELINE.json to time as well (2, 4, 5, 5skew); 'none' leaves them out")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the block-sparse products have no multi-GPU path in this build (--gpus must be 1)")
-    extra = [c for c in args.configs.split(",") if c]
+    extra = [c for c in args.configs.split(",") if c and c != "none"]
     for name in extra:
         if name not in ("2", "4", "5", "5skew"):
-            sys.exit(f"bench.py: unknown configuration {name!r} (2, 4, 5, 5skew)")
+            sys.exit(f"bench.py: unknown configuration {name!r} (2, 4, 5, 5skew, or none)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     import stk_amd as stk
@@ -335,19 +425,24 @@ def main():
     names = ("sdd", "dsd", "dds")
     state = {}
 
-    def step(events=None):
-        marks = []
-        if events is not None:
-            marks.append(events[0]); events[0].record()
+    def run_sdd():
         state["h"] = stk.ops.sdd(x, w1, topo)
-        if events is not None:
-            events[1].record()
+
+    def run_dsd():
         state["y"] = stk.ops.dsd(state["h"], w2)
-        if events is not None:
-            events[2].record()
+
+    def run_dds():
         state["dw1"] = stk.ops.dds(xt, state["h"])
+
+    products = (run_sdd, run_dsd, run_dds)
+
+    def step(events=None):
         if events is not None:
-            events[3].record()
+            events[0].record()
+        for i, product in enumerate(products):
+            product()
+            if events is not None:
+                events[i + 1].record()
 
     if args.copy_calibration:
         # one elementwise kernel (torch.neg) that reads 1 GiB and writes 1 GiB in a single dispatch
@@ -356,20 +451,50 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    aux_steps = max(10, args.steps // 2)
+
+    def preheat(ms):
+        """Untimed steps for `ms` milliseconds, without a pause at the end."""
+        t0, n = time.perf_counter(), 0
+        while (time.perf_counter() - t0) * 1e3 < ms:
+            for _ in range(5):
+                step()
+            torch.cuda.synchronize()
+            n += 5
+        return n
+
     with torch.no_grad():
+        step()
+        # the collector of Python objects stays out of the timed passes (a full collection stops the launches
+        # for tens of milliseconds, and the idle GPU drops its clocks); nothing in a step creates reference cycles
+        gc.collect()
+        gc.disable()
+        # untimed: the step itself until the clocks have settled; the comparators then run at the same clocks
+        preheat_steps = preheat(args.preheat_ms)
+        dense = dense_comparators(rows, dev, aux_steps, 5)
+        routing = routing_times(dev, aux_steps, 5)
+        preheat_steps += preheat(args.preheat_ms / 3)
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+
+        # the same K steps again with an event between the launches: duration of each kernel inside the step
         evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
         t0 = time.perf_counter()
         for i in range(args.steps):
             step(evs[i])
         torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-
+        wall_with_events = time.perf_counter() - t0
         per_op_ms = {n: float(np.mean([e[i].elapsed_time(e[i + 1]) for e in evs])) for i, n in enumerate(names)}
-        dense = dense_comparators(rows, dev, max(10, args.steps // 2), 5)
-        routing = routing_times(dev, max(10, args.steps // 2), 5)
+        # and each product on its own, back to back
+        per_op_b2b_ms = {n: time_batch(product, args.steps) for n, product in zip(names, products)}
+        gc.enable()
+
         others = {}
         for name in extra:
             others[name] = other_config(name, dev, max(5, args.steps // 2), 3)
@@ -379,6 +504,8 @@ def main():
     value = 3 * flops_op / (ms_per_step * 1e-3) / 1e12
     per_op_tflops = {n: flops_op / (per_op_ms[n] * 1e-3) / 1e12 for n in names}
     frac_dense = {n: per_op_tflops[n] / dense[n + "_like_tflops"] for n in names}
+    frac_dense_b2b = {n: dense[n + "_like_back_to_back_ms"] / per_op_b2b_ms[n] * (flops_op / (2.0 * EXPERTS * dense["tokens_per_expert"] * HIDDEN * FFN))
+                      for n in names}
     dense_total_ms = sum(dense[n + "_like_ms"] for n in names)
     dense_flops = 2.0 * EXPERTS * dense["tokens_per_expert"] * HIDDEN * FFN
     dense_step_tflops = 3 * dense_flops / (dense_total_ms * 1e-3) / 1e12
@@ -393,8 +520,12 @@ def main():
         achieved = per_op_tflops[dominant]
         roof = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS}
     kernel_names = {"sdd": "sdd_fused_kernel", "dsd": "dsd_sliced_kernel", "dds": "dds_fused_kernel"}
-    roof.update({"traffic": measured_hbm_traffic(kernel_names[dominant]), "kernel": kernel_names[dominant], "avg_launch_ms": per_op_ms[dominant],
-                 "algorithmic_bytes": bytes_op[dominant], "flops": flops_op})
+    traffic, traffic_source = measured_hbm_traffic(kernel_names[dominant])
+    roof.update({"traffic": traffic, "traffic_source": traffic_source, "kernel": kernel_names[dominant], "avg_launch_ms": per_op_ms[dominant],
+                 "algorithmic_bytes": bytes_op[dominant], "flops": flops_op,
+                 "per_kernel": {kernel_names[n]: {"avg_launch_ms": per_op_ms[n], "algorithmic_bytes": bytes_op[n],
+                                                  "frac_of_hbm_peak": bytes_op[n] / (per_op_ms[n] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                                  "traffic": measured_hbm_traffic(kernel_names[n])[0]} for n in names}})
 
     result = {
         "metric": "nonzero-block TFLOP/s for SDD/DSD/DDS; % of dense bf16 GEMM at dMoE shape",
@@ -404,9 +535,16 @@ def main():
         "config": {"workload": "dmoe_ffn_fwd_topology: 16384 tokens top-1 over 64 experts (seed 0) padded to 128, hidden 1024, "
                                "ffn 4096, blocking 128; step = sdd(x,W1) + dsd(h,W2) + dds(x^T,h)",
                    "nnz_blocks": int(nnz), "padded_tokens": int(rows), "flops_per_product": flops_op},
-        "per_op_ms": per_op_ms, "per_op_tflops": per_op_tflops,
+        "timing": "value and ms_per_step: wall clock over the K steps between two synchronisations, nothing but the launches inside; "
+                  "per_op_ms: a second pass of K steps with a HIP event between the launches (ms_per_step_with_events); "
+                  "per_op_back_to_back_ms: each product K times between one pair of events; before the W warm-up steps the "
+                  "dense comparators and the routing are timed and the step runs untimed for `preheat.ms` (clock ramp after idle)",
+        "preheat": {"ms": args.preheat_ms, "steps": preheat_steps},
+        "ms_per_step_with_events": wall_with_events * 1e3 / args.steps,
+        "per_op_ms": per_op_ms, "per_op_tflops": per_op_tflops, "per_op_back_to_back_ms": per_op_b2b_ms,
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
-        "dense": dense, "frac_of_dense_per_op": frac_dense, "frac_of_dense_step": value / dense_step_tflops,
+        "dense": dense, "frac_of_dense_per_op": frac_dense, "frac_of_dense_per_op_back_to_back": frac_dense_b2b,
+        "frac_of_dense_step": value / dense_step_tflops,
         "roofline": roof,
         "routing": routing,
     }

@@ -26,6 +26,12 @@
 #define STK_DDS_STAGES 4
 #endif
 
+// Large dense results (dsd, dds) are written with non-temporal stores, so that they do not displace the
+// operands from the caches.
+#ifndef STK_STREAM_STORES
+#define STK_STREAM_STORES true
+#endif
+
 namespace stk {
 
 // Per-thread message behind stk_last_error().

@@ -70,7 +70,7 @@ __device__ __forceinline__ void dds_tile(const DdsArgs& g, int bj, int m0, char*
   }
   const WaveCoords w = wave_coords<Cfg>();
   const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, true>(acc, g.out + (int64_t)(m0 + wm0) * g.ldc + (int64_t)bj * BLK + wn0, g.ldc, m_valid - wm0, Cfg::TN - wn0, smem);
+  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + (int64_t)(m0 + wm0) * g.ldc + (int64_t)bj * BLK + wn0, g.ldc, m_valid - wm0, Cfg::TN - wn0, smem);
 }
 
 // One block column per workgroup (four wavefronts).

@@ -74,7 +74,7 @@ __device__ __forceinline__ void dsd_store(f32x16_t (&acc)[Cfg::IM][Cfg::JN], con
   const int n_valid = (g.n - n0 < Cfg::TN) ? g.n - n0 : Cfg::TN;
   const WaveCoords w = wave_coords<Cfg>();
   const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, true>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, Cfg::TM - wm0, n_valid - wn0, smem);
+  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, Cfg::TM - wm0, n_valid - wn0, smem);
 }
 
 // The whole tile of LINES block rows starting at `bi`, output columns [n0, n0 + Cfg::TN).
