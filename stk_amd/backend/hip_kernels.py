@@ -271,7 +271,7 @@ def dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_ind
     assert data.is_contiguous() and out.stride(1) == 1
     assert data.dtype == rhs.dtype == out.dtype
     ci, cit = _index(column_indices), _index(column_indices_t)
-    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t) if FUSION and b == 128 and data.shape[0] > 0 else None
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b) if FUSION and b in (64, 128) and data.shape[0] > 0 else None
     with _on_device(out.device):
         ws = _dsd_workspace(out.device, m, n, b) if plan is not None else None
         status = _lib.load().stk_dsd(
@@ -300,7 +300,7 @@ def dds(lhs, shape, data, offsets, row_indices, column_indices, offsets_t, colum
     assert data.is_contiguous() and out.stride(1) == 1
     assert data.dtype == lhs.dtype == out.dtype
     ci, cit = _index(column_indices), _index(column_indices_t)
-    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t) if FUSION and b == 128 and data.shape[0] > 0 else None
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b) if FUSION and b in (64, 128) and data.shape[0] > 0 else None
     with _on_device(out.device):
         _lib.check(_lib.load().stk_dds(
             m, k, n, lhs.data_ptr(), lhs.stride(0), lhs.stride(1), data.data_ptr(),

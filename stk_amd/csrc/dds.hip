@@ -27,16 +27,17 @@ struct DdsArgs {
   int small;       // little work per compute unit: four-wave tiles
 };
 
-// LINES block columns starting at `bj` (identical patterns when LINES == 2), output
-// rows [m0, m0 + Cfg::TM).
+// LINES block columns starting at `bj` (identical patterns when LINES > 1), output
+// rows [m0, m0 + Cfg::TM).  Only the first `lines` of the LINES columns exist; the others are
+// computed on the last one's blocks and dropped.
 template <class Cfg, int BLK, bool TRANS_B, bool FULL, int LINES>
-__device__ __forceinline__ void dds_tile(const DdsArgs& g, int bj, int m0, char* smem) {
+__device__ __forceinline__ void dds_tile(const DdsArgs& g, int bj, int m0, char* smem, int lines = LINES) {
   static_assert(Cfg::TN == LINES * BLK && Cfg::B_PARTS == LINES && Cfg::B_KMAJOR == TRANS_B, "one operand part per block column");
   constexpr int KT = Cfg::KT;
   constexpr int kTilesPerBlock = BLK / KT;
   int start[LINES];
 #pragma unroll
-  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bj + l];
+  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bj + (l < lines ? l : lines - 1)];
   const int nseg = g.walk_offsets[bj + 1] - start[0];
   const elem_t* a0 = g.lhs + (int64_t)m0 * (Cfg::A_KMAJOR ? g.lda : 1);
   const int64_t a_kstride = Cfg::A_KMAJOR ? 1 : g.lda;
@@ -70,7 +71,7 @@ __device__ __forceinline__ void dds_tile(const DdsArgs& g, int bj, int m0, char*
   }
   const WaveCoords w = wave_coords<Cfg>();
   const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + (int64_t)(m0 + wm0) * g.ldc + (int64_t)bj * BLK + wn0, g.ldc, m_valid - wm0, Cfg::TN - wn0, smem);
+  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + (int64_t)(m0 + wm0) * g.ldc + (int64_t)bj * BLK + wn0, g.ldc, m_valid - wm0, lines * BLK - wn0, smem);
 }
 
 // One block column per workgroup (four wavefronts).
@@ -80,6 +81,49 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dds_kernel(DdsArgs g) {
   const int ntm = (g.m + Cfg::TM - 1) / Cfg::TM;
   const int item = xcd_grouped(blockIdx.x, g.block_cols * ntm);  // no plan, no hint about the lines: small groups
   dds_tile<Cfg, BLK, TRANS_B, FULL, 1>(g, item / ntm, (item % ntm) * Cfg::TM, smem);
+}
+
+// The lone block columns of a plan's list, one per workgroup (four wavefronts): what dds_fused64_kernel leaves.
+template <class Cfg, int BLK, bool TRANS_B, bool FULL>
+__global__ __launch_bounds__(Cfg::kThreads, 2) void dds_singles_kernel(DdsArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  const int ntm = (g.m + Cfg::TM - 1) / Cfg::TM;
+  const int tiles = const_ints(plan.counts)[kTallSingles] * ntm;
+  if ((int)blockIdx.x >= tiles) return;
+  const int item = xcd_grouped(blockIdx.x, tiles);
+  dds_tile<Cfg, BLK, TRANS_B, FULL, 1>(g, const_ints(plan.list(kTallSingles))[item / ntm], (item % ntm) * Cfg::TM, smem);
+}
+
+// 64-blocks with a plan built for them, eight wavefronts: groups of four identical block columns as 256x256
+// tiles (a group of three runs on the same shape with its fourth column dropped), pairs as 256x128 tiles; the
+// dense operand is then read once per 256 or 128 columns instead of once per 64.  Lone columns are left to
+// dds_singles_kernel.  The grid is an upper bound; the surplus leaves at once.
+template <class Quad, class Pair, bool TRANS_B>
+__global__ __launch_bounds__(512, 2) void dds_fused64_kernel(DdsArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  static_assert(Quad::TM == Pair::TM, "same row tiling");
+  const int ntm = g.m / Quad::TM;
+  const int quad_tiles = const_ints(plan.counts)[kPairs] * ntm, triple_tiles = const_ints(plan.counts)[kTallTriples] * ntm;
+  const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntm;
+  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
+  int bid = blockIdx.x;
+  // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
+  if (bid < pair_tiles) {
+    const int item = xcd_item(bid, pair_tiles, spread);
+    dds_tile<Pair, 64, TRANS_B, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntm], (item % ntm) * Pair::TM, smem, 2);
+    return;
+  }
+  bid -= pair_tiles;
+  if (bid < quad_tiles) {
+    const int item = xcd_item(bid, quad_tiles, spread);
+    dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Quad::TM, smem, 4);
+    return;
+  }
+  bid -= quad_tiles;
+  if (bid < triple_tiles) {
+    const int item = xcd_item(bid, triple_tiles, spread);
+    dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntm], (item % ntm) * Quad::TM, smem, 3);
+  }
 }
 
 // 128-blocks, eight wavefronts: 256x256 tiles over the pairs of identical block columns, then
@@ -150,6 +194,19 @@ static void launch_dds(const DdsArgs& g, const PlanLists& plan, hipStream_t stre
   } else {
     // 64-blocks: 4x1 wavefronts of 64x64 (tile 256x64)
     using Dma = TileCfg<4, 1, 2, 2, 1, 1, 1, AK, TRANS_B, BF16, 64, 2, STREAM>;
+    if (plan.counts && g.m % 256 == 0 && !g.small) {
+      // groups of identical block columns on eight wavefronts (4x2 of 64x128 over four block columns, 4x2 of 64x64
+      // over two), then the lone columns one per four-wave workgroup; both grids are upper bounds
+      using Quad = TileCfg<4, 2, 2, 4, 1, 2, 4, AK, TRANS_B, BF16, 64, 2, STREAM>;
+      using Pair = TileCfg<4, 2, 2, 2, 1, 2, 2, AK, TRANS_B, BF16, 64, 2, STREAM>;
+      constexpr int lds = Quad::kSmemBytes > Pair::kSmemBytes ? Quad::kSmemBytes : Pair::kSmemBytes;
+      static const int once = (set_lds_limit(&dds_fused64_kernel<Quad, Pair, TRANS_B>, lds), set_lds_limit(&dds_singles_kernel<Dma, 64, TRANS_B, true>, Dma::kSmemBytes), 0);
+      (void)once;
+      const int ntm = g.m / 256;
+      hipLaunchKernelGGL((dds_fused64_kernel<Quad, Pair, TRANS_B>), dim3((g.block_cols + 1) / 2 * ntm), dim3(512), lds, stream, g, plan);
+      hipLaunchKernelGGL((dds_singles_kernel<Dma, 64, TRANS_B, true>), dim3(g.block_cols * ntm), dim3(Dma::kThreads), Dma::kSmemBytes, stream, g, plan);
+      return;
+    }
     if (g.m % Dma::TM == 0) launch_one<Dma, BLK, TRANS_B, true>(g, stream);
     else launch_one<Dma, BLK, TRANS_B, false>(g, stream);
   }

@@ -28,15 +28,17 @@ struct DsdArgs {
 };
 
 // acc += the products of walk entries [e0, e1) of LINES block rows starting at `bi` (identical
-// patterns when LINES > 1) with output columns [n0, n0 + Cfg::TN).
+// patterns when LINES > 1) with output columns [n0, n0 + Cfg::TN).  Only the first `lines` of the
+// LINES rows exist; the others are computed on the last one's blocks and dropped by the caller.
 template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES>
-__device__ __forceinline__ void dsd_accumulate(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, int e0, int e1, char* smem) {
+__device__ __forceinline__ void dsd_accumulate(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, int e0, int e1, char* smem,
+                                               int lines = LINES) {
   static_assert(Cfg::TM == LINES * BLK && Cfg::A_PARTS == LINES && Cfg::A_KMAJOR == !TRANS_A, "one operand part per block row");
   constexpr int KT = Cfg::KT;
   constexpr int kTilesPerBlock = BLK / KT;
   int start[LINES];
 #pragma unroll
-  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bi + l];
+  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bi + (l < lines ? l : lines - 1)];
   const elem_t* b0 = g.rhs + (int64_t)n0 * (Cfg::B_KMAJOR ? g.ldb : 1);
   const int64_t b_kstride = Cfg::B_KMAJOR ? 1 : g.ldb;
   const int64_t b_part = (int64_t)Cfg::PN * (Cfg::B_KMAJOR ? g.ldb : 1);
@@ -68,21 +70,22 @@ __device__ __forceinline__ void dsd_accumulate(f32x16_t (&acc)[Cfg::IM][Cfg::JN]
   }
 }
 
-// Writes the finished tile: rows of block row `bi` onwards, columns from n0.
+// Writes the finished tile: the first `rows` rows from block row `bi` onwards, columns from n0.
 template <class Cfg, int BLK>
-__device__ __forceinline__ void dsd_store(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, char* smem) {
+__device__ __forceinline__ void dsd_store(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, char* smem, int rows = Cfg::TM) {
   const int n_valid = (g.n - n0 < Cfg::TN) ? g.n - n0 : Cfg::TN;
   const WaveCoords w = wave_coords<Cfg>();
   const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, Cfg::TM - wm0, n_valid - wn0, smem);
+  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, rows - wm0, n_valid - wn0, smem);
 }
 
-// The whole tile of LINES block rows starting at `bi`, output columns [n0, n0 + Cfg::TN).
+// The whole tile of LINES block rows starting at `bi` (the first `lines` of them exist), output columns
+// [n0, n0 + Cfg::TN).
 template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES>
-__device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char* smem) {
+__device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char* smem, int lines = LINES) {
   f32x16_t acc[Cfg::IM][Cfg::JN] = {};
-  dsd_accumulate<Cfg, BLK, TRANS_A, FULL, LINES>(acc, g, bi, n0, 0, g.walk_offsets[bi + 1] - g.walk_offsets[bi], smem);
-  dsd_store<Cfg, BLK>(acc, g, bi, n0, smem);
+  dsd_accumulate<Cfg, BLK, TRANS_A, FULL, LINES>(acc, g, bi, n0, 0, g.walk_offsets[bi + 1] - g.walk_offsets[bi], smem, lines);
+  dsd_store<Cfg, BLK>(acc, g, bi, n0, smem, lines * BLK);
 }
 
 // One block row per workgroup (four wavefronts).
@@ -92,6 +95,49 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_kernel(DsdArgs g) {
   const int ntn = (g.n + Cfg::TN - 1) / Cfg::TN;
   const int item = xcd_grouped(blockIdx.x, g.block_rows * ntn);  // no plan, no hint about the lines: small groups
   dsd_tile<Cfg, BLK, TRANS_A, FULL, 1>(g, item / ntn, (item % ntn) * Cfg::TN, smem);
+}
+
+// The lone block rows of a plan's list, one per workgroup (four wavefronts): what dsd_fused64_kernel leaves.
+template <class Cfg, int BLK, bool TRANS_A, bool FULL>
+__global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_singles_kernel(DsdArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  const int ntn = (g.n + Cfg::TN - 1) / Cfg::TN;
+  const int tiles = const_ints(plan.counts)[kTallSingles] * ntn;
+  if ((int)blockIdx.x >= tiles) return;
+  const int item = xcd_grouped(blockIdx.x, tiles);
+  dsd_tile<Cfg, BLK, TRANS_A, FULL, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Cfg::TN, smem);
+}
+
+// 64-blocks with a plan built for them, eight wavefronts: groups of four identical block rows as 256x256
+// tiles (a group of three runs on the same shape with its fourth row dropped), pairs as 128x256 tiles; the dense
+// operand is then read once per 256 or 128 rows instead of once per 64.  Lone rows are left to
+// dsd_singles_kernel.  The grid is an upper bound; the surplus leaves at once.
+template <class Quad, class Pair, bool TRANS_A>
+__global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  static_assert(Quad::TN == Pair::TN, "same column tiling");
+  const int ntn = g.n / Quad::TN;
+  const int quad_tiles = const_ints(plan.counts)[kPairs] * ntn, triple_tiles = const_ints(plan.counts)[kTallTriples] * ntn;
+  const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
+  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
+  int bid = blockIdx.x;
+  // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
+  if (bid < pair_tiles) {
+    const int item = xcd_item(bid, pair_tiles, spread);
+    dsd_tile<Pair, 64, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Pair::TN, smem, 2);
+    return;
+  }
+  bid -= pair_tiles;
+  if (bid < quad_tiles) {
+    const int item = xcd_item(bid, quad_tiles, spread);
+    dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kPairs))[item / ntn], (item % ntn) * Quad::TN, smem, 4);
+    return;
+  }
+  bid -= quad_tiles;
+  if (bid < triple_tiles) {
+    const int item = xcd_item(bid, triple_tiles, spread);
+    dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntn], (item % ntn) * Quad::TN, smem, 3);
+  }
 }
 
 // 128-blocks, eight wavefronts.  The workgroups take their tiles from the lists of the plan,
@@ -365,6 +411,19 @@ static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* 
   } else {
     // 64-blocks: 1x4 wavefronts of 64x64 (tile 64x256)
     using Dma = TileCfg<1, 4, 2, 2, 1, 1, 1, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
+    if (plan.counts && g.n % 256 == 0 && !g.small) {
+      // groups of identical block rows on eight wavefronts (4x2 of 64x128 over four block rows, 2x4 of 64x64 over
+      // two), then the lone rows one per four-wave workgroup; both grids are upper bounds
+      using Quad = TileCfg<4, 2, 2, 4, 1, 4, 2, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
+      using Pair = TileCfg<2, 4, 2, 2, 1, 2, 2, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
+      constexpr int lds = Quad::kSmemBytes > Pair::kSmemBytes ? Quad::kSmemBytes : Pair::kSmemBytes;
+      static const int once = (set_lds_limit(&dsd_fused64_kernel<Quad, Pair, TRANS_A>, lds), set_lds_limit(&dsd_singles_kernel<Dma, 64, TRANS_A, true>, Dma::kSmemBytes), 0);
+      (void)once;
+      const int ntn = g.n / 256;
+      hipLaunchKernelGGL((dsd_fused64_kernel<Quad, Pair, TRANS_A>), dim3((g.block_rows + 1) / 2 * ntn), dim3(512), lds, stream, g, plan);
+      hipLaunchKernelGGL((dsd_singles_kernel<Dma, 64, TRANS_A, true>), dim3(g.block_rows * ntn), dim3(Dma::kThreads), Dma::kSmemBytes, stream, g, plan);
+      return;
+    }
     if (g.n % Dma::TN == 0) launch_one<Dma, BLK, TRANS_A, true>(g, stream);
     else launch_one<Dma, BLK, TRANS_A, false>(g, stream);
   }

@@ -23,6 +23,17 @@
 // operand has 256 (t + 1) columns, t = 0 .. 15 (1: not at all).  The plan depends on the
 // topology (and on the number of compute units of the device it is built on) only, so
 // callers may build it once and reuse it for every product on that topology.
+//
+// A plan built for blocking 64 groups the lines by fours instead (stk_dsd and stk_dds then compute up to four
+// identical lines as one 256-wide tile): a run of identical lines is cut from its start into fours while they
+// last, and the three, two or one lines that are left form one more group.  Lines so long that a tile over four
+// of them would be more than a compute unit's share of the whole product (four times their blocks exceed
+// 4 nnz / compute units: the expert that takes half of the tokens of a skewed routing) are cut into pairs
+// instead, which the kernels start first.  Both role arrays then hold, for the
+// first line of a group, the number of its lines (0 for the other lines), and the lists are
+//   list 0 (role 1's place)  first lines of groups of four      list 3 (tall 3's place)  of groups of three
+//   list 2 (tall 1's place)  of pairs                           list 4 (tall 0's place)  lone lines
+// with list 1 empty.
 #include "common.h"
 
 namespace stk {
@@ -157,6 +168,19 @@ __device__ __forceinline__ int sdd_rows_owned(const uint8_t* same, int i, int po
   if (q == 0) return left;                  // a pair or a single line
   return 0;
 }
+// The same for the groups of stk_dsd / stk_dds with 64-blocks: fours (as above) unless the lines are `heavy`, then
+// pairs from the start of the run with a lone line left over when its length is odd.
+__device__ __forceinline__ int lines_owned64(const uint8_t* same, int i, int pos, bool heavy) {
+  if (!heavy) return sdd_rows_owned(same, i, pos, 4);
+  if (pos & 1) return 0;
+  return same[i] ? 2 : 1;
+}
+// A tile over four lines of `blocks` blocks each would be more than a compute unit's share of a product whose
+// other dimension has four tiles.
+__device__ __forceinline__ bool heavy_line(int blocks, int64_t nnz, int compute_units) {
+  const int64_t share = nnz * 4 / (compute_units > 0 ? compute_units : 1);
+  return 4 * (int64_t)blocks > (share > 1 ? share : 1);
+}
 // Blocks side by side in the tiles of a group of `rows` lines.
 // (most_cols == 2: a group of three rows has tiles of 3 x 1 blocks; most_cols == 4: every tile is up to four wide)
 __device__ __forceinline__ int sdd_cols_of(int rows, int most_cols) { return (rows == 3 && most_cols == 2) ? 1 : most_cols; }
@@ -166,7 +190,7 @@ __device__ __forceinline__ int sdd_cols_of(int rows, int most_cols) { return (ro
 __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restrict__ offsets, int block_rows,
                                                           const int32_t* __restrict__ offsets_t, int block_cols,
                                                           int compute_units, uint8_t* __restrict__ plan, int32_t* __restrict__ sdd, int max_sdd_tiles,
-                                                          int sdd_rows, int sdd_cols) {
+                                                          int sdd_rows, int sdd_cols, int most) {
   __shared__ int wave_last[16];
   __shared__ float sim_time[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
   __shared__ int sim_count[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
@@ -207,6 +231,17 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
   for (int i = lo; i < hi; i++) {
     if (i == 0 || same[i - 1] == 0) start = i;
     const int pos = i - start;
+    if (most == 4) {
+      // groups of up to four lines: the first line of a group holds the group's size
+      const int32_t* offs = cols ? offsets_t : offsets;
+      const int n = lines_owned64(same, i, pos, heavy_line(offs[i + 1] - offs[i], offs[lines], compute_units));
+      role[i] = tall[i] = (uint8_t)n;
+      mine[kPairs] += n == 4;
+      mine[kTallTriples] += n == 3;
+      mine[kTallPairs] += n == 2;
+      mine[kTallSingles] += n == 1;
+      continue;
+    }
     const int r = (pos & 1) ? 2 : (same[i] ? 1 : 0);
     int t = 2;  // odd positions, and the last line of an odd run of three or more, are covered
     if ((pos & 1) == 0) {
@@ -244,7 +279,8 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
     if (tid == 0) lists[(cols ? kPlanLists : 0) + kind] = total;
     totals[kind] = total;
     const uint8_t* from = kind < 2 ? role : tall;
-    const int want = kind == 0 ? 1 : kind == 1 ? 0 : kind == 2 ? 1 : kind == 3 ? 3 : 0;
+    int want = kind == 0 ? 1 : kind == 1 ? 0 : kind == 2 ? 1 : kind == 3 ? 3 : 0;
+    if (most == 4) want = kind == kPairs ? 4 : kind == kTallTriples ? 3 : kind == kTallPairs ? 2 : kind == kTallSingles ? 1 : -1;
     for (int i = lo; i < hi; i++)
       if (from[i] == want) list[base++] = i;
   }
@@ -362,6 +398,6 @@ extern "C" int stk_build_plan(const int32_t* offsets, const void* column_indices
     hipLaunchKernelGGL((plan_same_kernel<int16_t>), dim3(grid), dim3(256), 0, s, offsets, static_cast<const int16_t*>(column_indices),
                        (int)block_rows, offsets_t, static_cast<const int16_t*>(column_indices_t), (int)block_cols, plan);
   hipLaunchKernelGGL(plan_roles_kernel, dim3(2), dim3(1024), 0, s, offsets, (int)block_rows, offsets_t, (int)block_cols, compute_units(), plan, sdd,
-                     (int)sdd_max_tiles(block_rows, nnz), blocking == 64 ? 4 : 2, blocking == 64 ? 4 : 2);
+                     (int)sdd_max_tiles(block_rows, nnz), blocking == 64 ? 4 : 2, blocking == 64 ? 4 : 2, blocking == 64 ? 4 : 2);
   return check_launch("stk_build_plan");
 }

@@ -375,14 +375,16 @@ def test_dmoe_small_against_oracle(blocking, dtype):
     U.assert_close(dw2, O.dsd((topo.shape[1], topo.shape[0]), U.np32(h.data), topo, True, U.np32(x)), dtype, "dmoe dsd t")
 
 
+@pytest.mark.parametrize("b", [128, 64])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hidden", [256, 2048])
-def test_dsd_runs_of_identical_rows(hidden, dtype):
+def test_dsd_runs_of_identical_rows(hidden, dtype, b):
     # block rows in runs of 1..7 identical rows (and an expert without tokens): pairs become 256-row
     # tiles, the last three rows of an odd run one 384-row tile; the dense operand also as a .t() view.
     # (hidden 256: little work per compute unit, which runs on four-wave 128x128 tiles instead)
-    tokens = np.array([128, 256, 0, 384, 512, 640, 768, 896, 100])
-    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden, 4096, 128, dtype, 5)
+    # With 64-blocks the same token counts give runs of 2..14 rows (and one of 1): fours, threes, pairs, a lone row.
+    tokens = np.array([128, 256, 0, 384, 512, 640, 768, 896, 100, 60])
+    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden, 4096, b, dtype, 5)
     g = torch.Generator().manual_seed(11)
     h = stk.Matrix(tm.size(), (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV), tm.row_indices, tm.column_indices, tm.offsets)
     want = O.dsd(topo.shape, U.np32(h.data), topo, False, U.np32(w2))
@@ -391,9 +393,13 @@ def test_dsd_runs_of_identical_rows(hidden, dtype):
     U.assert_close(stk.ops.dsd(h, w2t.t()), want, dtype, "dsd runs, transposed view")
     # identical columns walked through the transpose metadata: three block columns per expert
     tokens = np.array([300, 128, 650]) if hidden == 256 else np.array([3000, 1280, 6500, 2000, 4000])
-    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden if hidden == 256 else 4096, 384, 128, dtype, 6)
+    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden if hidden == 256 else 4096, 384, b, dtype, 6)
     h = stk.Matrix(tm.size(), (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV), tm.row_indices, tm.column_indices, tm.offsets)
     U.assert_close(stk.ops.dsd(h.t(), x), O.dsd((topo.shape[1], topo.shape[0]), U.np32(h.data), topo, True, U.np32(x)), dtype, "dsd t, runs of three columns")
+    # dds over the same runs: identical block columns (three or six per expert) and, transposed, identical block rows
+    U.assert_close(stk.ops.dds(x.t(), h), O.dds(U.np32(x).T, topo.shape, U.np32(h.data), topo, False), dtype, "dds, runs of columns")
+    v = _dense(256, topo.shape[1], dtype, 0.05).detach()
+    U.assert_close(stk.ops.dds(v, h.t()), O.dds(U.np32(v), (topo.shape[1], topo.shape[0]), U.np32(h.data), topo, True), dtype, "dds t, runs of rows")
 
 
 @pytest.mark.parametrize("b", [128, 64])
@@ -450,26 +456,34 @@ def test_lines_longer_than_the_lane_resident_walk_table(blocks):
     U.assert_close(stk.ops.dsd(st.t(), x), O.dsd((rows, cols), U.np32(st.data), topo_t, True, U.np32(x)), dtype, "dsd t long columns")
 
 
-def test_results_do_not_depend_on_the_fusion_plan(monkeypatch):
-    # identical rows / columns computed as fused tiles (pairs, threes) or one line at a time: every output
-    # element accumulates its k-steps in the same order, so the results are equal bit for bit (as long as dsd
-    # does not cut tiles along k, which needs its workspace)
+@pytest.mark.parametrize("b", [128, 64])
+def test_results_do_not_depend_on_the_fusion_plan(monkeypatch, b):
+    # identical rows / columns computed as fused tiles (pairs, threes; fours with 64-blocks) or one line at a time:
+    # every output element accumulates its k-steps in the same order, so the results are equal bit for bit (as long
+    # as dsd does not cut tiles along k, which needs its workspace)
     from stk_amd.backend import hip_kernels
     monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
     dtype = torch.bfloat16
-    tokens = np.array([300, 0, 129, 384, 640, 128, 77, 256])
-    topo, tm, x, w1, w2 = _dmoe_case(tokens, 4096, 4096, 128, dtype, 9)    # enough work for the fused tiles of all three
+    tokens = np.array([300, 0, 129, 384, 640, 128, 77, 256, 40])
+    topo, tm, x, w1, w2 = _dmoe_case(tokens, 4096, 4096, b, dtype, 9)    # enough work for the fused tiles of all three
+
+    h0 = stk.ops.sdd(x, w1, tm)
 
     def run():
         h = stk.ops.sdd(x, w1, tm)
-        return h.data.clone(), stk.ops.dsd(h, w2), stk.ops.dds(x.t(), h), stk.ops.dsd(h.t(), x), stk.ops.dds(w1, h.t())
+        return h.data.clone(), stk.ops.dsd(h0, w2), stk.ops.dds(x.t(), h0), stk.ops.dsd(h0.t(), x), stk.ops.dds(w1, h0.t())
 
     fused = run()
     monkeypatch.setattr(hip_kernels, "FUSION", False)
     plain = run()
-    for a, b, what in zip(fused, plain, ("sdd", "dsd", "dds", "dsd t", "dds t")):
-        assert torch.equal(a, b), what
-    U.assert_close(plain[1], O.dsd(topo.shape, U.np32(plain[0]), topo, False, U.np32(w2)), dtype, "dsd without plan")
+    for a, c, what in zip(fused, plain, ("sdd", "dsd", "dds", "dsd t", "dds t")):
+        if what == "sdd" and b == 64:
+            # without a plan a 64-block is computed with k split over the four wavefronts of its workgroup and the
+            # partial sums added at the end: the same sums in another order
+            U.assert_close_scaled(a, c.float(), dtype, "sdd, 64-blocks with and without a plan")
+        else:
+            assert torch.equal(a, c), what
+    U.assert_close(plain[1], O.dsd(topo.shape, U.np32(h0.data), topo, False, U.np32(w2)), dtype, "dsd without plan")
 
 
 def test_gradients_side_by_side_equal_gradients_one_after_the_other(monkeypatch):

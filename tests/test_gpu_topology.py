@@ -259,9 +259,44 @@ def test_fusion_plan_roles(name):
     plan64 = hip_kernels.fusion_plan(_dev(topo.offsets.copy()), _dev(topo.column_indices), blocking=64).cpu().numpy()
     sdd64 = plan64[:8 + 8 * max_tiles].view(np.int32)
     assert sdd64[2:2 + 2 * sdd64[0]].reshape(-1, 2).tolist() == _sdd_tiles(topo.offsets, topo.column_indices, 4, 4)
+    # a plan for 64-blocks built with both directions: groups of up to four identical lines; both role arrays hold
+    # the size of the group at its first line, and the lists are fours, (none), pairs, threes, lone lines
+    both64 = hip_kernels.fusion_plan(_dev(topo.offsets.copy()), _dev(topo.column_indices), _dev(topo.offsets_t), _dev(topo.column_indices_t),
+                                     blocking=64).cpu().numpy()[sdd_bytes:]
+    want_rows, want_cols = _groups_of_up_to_four(topo.offsets, topo.column_indices), _groups_of_up_to_four(topo.offsets_t, topo.column_indices_t)
+    assert both64[:br].tolist() == want_rows and both64[br:br + bc].tolist() == want_cols
+    assert both64[2 * (br + bc):2 * (br + bc) + br].tolist() == want_rows
+    lists64 = both64[off:off + 4 * 5 * (2 + br + bc)].view(np.int32)
+    for d, (lines, sizes) in enumerate([(br, np.array(want_rows)), (bc, np.array(want_cols))]):
+        base = 10 + (5 * br if d else 0)
+        for kind, size in enumerate([4, None, 2, 3, 1]):
+            expect = [] if size is None else np.nonzero(sizes == size)[0].tolist()
+            assert int(lists64[5 * d + kind]) == len(expect), (d, kind)
+            assert lists64[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
     rows_only = hip_kernels.fusion_plan(_dev(topo.offsets), _dev(topo.column_indices)).cpu().numpy()
     assert rows_only[:8 + 8 * int(sdd[0])].tolist() == whole[:8 + 8 * int(sdd[0])].tolist()
     assert rows_only[sdd_bytes:sdd_bytes + br].tolist() == got[:br].tolist()
+
+
+def _groups_of_up_to_four(offsets, indices):
+    """Size of the group that starts at each line (0 for a line inside a group): a run of identical, non-empty
+    lines is cut from its start into fours while they last; the three, two or one lines left form one more group.
+    Lines with more than nnz / compute units blocks (a tile over four of them would exceed a compute unit's share
+    of a product with four tiles in the other dimension) are cut into pairs instead."""
+    lines = len(offsets) - 1
+    seg = [tuple(indices[offsets[i]:offsets[i + 1]]) for i in range(lines)]
+    share = max(1, int(offsets[lines]) * 4 // torch.cuda.get_device_properties(0).multi_processor_count)
+    size = [0] * lines
+    i = 0
+    while i < lines:
+        n = 1
+        while i + n < lines and len(seg[i]) > 0 and seg[i + n] == seg[i]:
+            n += 1
+        most = 2 if 4 * len(seg[i]) > share else 4
+        for a in range(0, n, most):
+            size[i + a] = min(most, n - a)
+        i += n
+    return size
 
 
 def _sdd_tiles(offsets, indices, most_rows, most_cols):
