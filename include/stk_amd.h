@@ -81,6 +81,9 @@ int stk_abi_version(void);
  * own a tile (per direction: role 1, role 0, and with groups of three 1, 3, 0), from which
  * stk_dsd and stk_dds take their work (with blocking 128), and 2 x 32 bytes of hints for
  * their launches.
+ * A plan built with blocking 64 groups the lines by fours instead of pairs (lists: first lines of groups of four,
+ * none, of pairs, of groups of three, lone lines; lines too long for a compute unit's share are cut into pairs); a
+ * plan must be passed only to products with the blocking it was built with.
  * Rb / Cb / nnz must be those of the stored matrix whenever the plan is passed to a
  * product (stk_sdd reads the tiles only and also accepts a plan built with Cb = 0).
  * The products accept plan == NULL (no fusion); results do not depend on it.
@@ -195,6 +198,26 @@ int stk_dds(int64_t m, int64_t k, int64_t n,
             int transpose_b,
             void* out, int64_t out_stride_m,
             int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
+
+/*
+ * Both operand gradients of a sampled product S = lhs * rhs in one call.  With the incoming gradient dS given as the
+ * values `data` of a matrix [m, k] with S's topology,
+ *   out_dsd [m, n_dsd]  = S [m, k] * rhs [k, n_dsd]        the gradient with respect to lhs (rhs here = rhs^T there)
+ *   out_dds [m_dds, k]  = lhs [m_dds, m] * S [m, k]        the gradient with respect to rhs (lhs here = lhs^T there)
+ * Replaces the pair of backend calls in SDD.backward, stk/backend/sputnik.py:274-299 (dsd at :280-288, dds at
+ * :289-297), which read dS twice in two launches.  With blocking 128, a plan, rhs as a .t() view of a row-major
+ * [n_dsd, k] and lhs as a .t() view of a row-major [m, m_dds] (what the backward pass of a product of two
+ * row-major operands passes), n_dsd and m_dds multiples of 256, both products run as one grid: the long tiles of
+ * the dsd first, the short tiles of the dds behind them.  Any other case runs stk_dsd (without a workspace) and
+ * then stk_dds.  Either way the results are those of stk_dsd without a workspace and of stk_dds, bit for bit.
+ * Arguments as for stk_dsd and stk_dds with transpose flags 0.
+ */
+int stk_dsd_dds(int64_t m, int64_t k,
+                const void* data, const int32_t* offsets, const void* column_indices,
+                const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                int64_t n_dsd, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, void* out_dsd, int64_t out_dsd_stride,
+                int64_t m_dds, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k, void* out_dds, int64_t out_dds_stride,
+                int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
 
 /*
  * COO block-row index from CSR offsets: out[offsets[r] .. offsets[r+1]) = r.

@@ -32,6 +32,8 @@ SIGNATURES = {
     "stk_dsd_tail_slices": (_int, [_i64, _i64, _i64, ctypes.c_double, _int]),
     "stk_dsd": (_int, [_i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _int, _p, _p, _i64, _p]),
     "stk_dds": (_int, [_i64, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _int, _int, _int, _p, _p]),
+    "stk_dsd_dds": (_int, [_i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64,
+                           _i64, _int, _int, _int, _p, _p]),
     "stk_row_indices": (_int, [_p, _i64, _i64, _p, _int, _p]),
     "stk_transpose_meta_workspace_bytes": (_sz, [_i64]),
     "stk_transpose_meta": (_int, [_p, _p, _i64, _i64, _int, _p, _p, _p, _p, _sz, _p]),

@@ -170,10 +170,21 @@ class DDS(torch.autograd.Function):
         return dlhs, None, ddata, None, None, None, None, None, None, None
 
 
+# Both gradients of sdd in one launch (stk_dsd_dds) where the operands' layouts allow it, instead of two launches
+# side by side; the same results.
+JOINT_GRADIENTS = True
+
+
 def _sdd_operand_gradients(ctx, lhs, rhs, sp, ds):
     """Gradients of S = lhs rhs (on the pattern) with respect to lhs and rhs, given dS as the values `ds`."""
     want_lhs = want_rhs = None
     lhs_is_view, rhs_is_view = _is_transposed_view(lhs), _is_transposed_view(rhs)
+    if JOINT_GRADIENTS and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and not rhs_is_view:
+        # dS rhs^T and lhs^T dS read the same dS: one call (sputnik.py:274-299 makes two)
+        dlhs = torch.empty((sp.shape[0], rhs.size(0)), dtype=lhs.dtype, device=lhs.device)
+        drhs = torch.empty((lhs.size(1), sp.shape[1]), dtype=rhs.dtype, device=rhs.device)
+        backend.dsd_dds(sp.shape, ds, *sp.meta, rhs.t(), dlhs, lhs.t(), drhs)
+        return dlhs, drhs
     if ctx.needs_input_grad[0]:
         if lhs_is_view:
             want_lhs = lambda: _run_dds(rhs, sp, ds, True)              # rhs dS^T, returned transposed

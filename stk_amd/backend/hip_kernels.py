@@ -310,6 +310,31 @@ def dds(lhs, shape, data, offsets, row_indices, column_indices, offsets_t, colum
             plan.data_ptr() if plan is not None else None, _stream()))
 
 
+def dsd_dds(shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t, rhs, out_dsd, lhs, out_dds):
+    """out_dsd = sparse @ rhs and out_dds = lhs @ sparse for one sparse operand [m, k] = `shape`, in one launch where
+    the layouts allow it (the two gradients of sdd, stk/backend/sputnik.py:274-299); otherwise the two products one
+    after the other.  The results are those of dsd (without its workspace) and dds, bit for bit."""
+    _need_gpu(data, rhs, lhs, out_dsd, out_dds)
+    m, k = shape
+    assert rhs.shape[0] == k and lhs.shape[1] == m, "incompatible dimensions"
+    b = _blocking(data)
+    _validate_matmul_dims(m, k, rhs.shape[1], b)
+    _validate_matmul_dims(lhs.shape[0], m, k, b)
+    rhs, lhs = _dense_operand(rhs), _dense_operand(lhs)
+    data = data.detach()
+    assert data.is_contiguous() and out_dsd.stride(1) == 1 and out_dds.stride(1) == 1
+    assert data.dtype == rhs.dtype == lhs.dtype == out_dsd.dtype == out_dds.dtype
+    ci, cit = _index(column_indices), _index(column_indices_t)
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b) if FUSION and b in (64, 128) and data.shape[0] > 0 else None
+    with _on_device(out_dsd.device):
+        _lib.check(_lib.load().stk_dsd_dds(
+            m, k, data.data_ptr(), _offsets(offsets).data_ptr(), ci.data_ptr(),
+            _offsets(offsets_t).data_ptr(), cit.data_ptr(), _offsets(block_offsets_t).data_ptr(),
+            rhs.shape[1], rhs.data_ptr(), rhs.stride(0), rhs.stride(1), out_dsd.data_ptr(), out_dsd.stride(0),
+            lhs.shape[0], lhs.data_ptr(), lhs.stride(0), lhs.stride(1), out_dds.data_ptr(), out_dds.stride(0),
+            data.shape[0], b, _value_dtype(data), _INDEX_DTYPES[ci.dtype], plan.data_ptr() if plan is not None else None, _stream()))
+
+
 def row_indices(shape, data, offsets, column_indices, out):
     """out[offsets[r]:offsets[r+1]] = r for every block row r."""
     _need_gpu(offsets, out)

@@ -108,6 +108,12 @@ inline int compute_units() {
   return cus;
 }
 
+// Kernels whose tiles need more dynamic LDS than the default limit say so once.
+template <class Kernel>
+inline void set_lds_limit(Kernel kernel, int bytes) {
+  if (bytes > 60000) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 // Read-only metadata read through the constant address space: wave-uniform loads become scalar loads.
 typedef const __attribute__((address_space(4))) int32_t* cint_t;
 __device__ __forceinline__ cint_t const_ints(const void* p) { return (cint_t)(uintptr_t)p; }

@@ -5,74 +5,9 @@
 // patterns, which then share every tile of the dense operand.  It walks the CSC
 // column segment of the sparse operand (for a transposed sparse operand: the CSR
 // row with direct block ids).
-#include "common.h"
-#include "gemm_core.h"
+#include "dds_tile.h"
 
 namespace stk {
-
-constexpr int kMaxSegments = 64;  // walk entries held at a time, one per lane of every wavefront
-
-struct DdsArgs {
-  const elem_t* lhs;
-  int64_t lda;
-  const elem_t* data;
-  const int32_t* walk_offsets;
-  const void* walk_columns;
-  const int32_t* walk_blocks;  // indirect block ids (non-transposed operand) or null
-  elem_t* out;
-  int64_t ldc;
-  int m;
-  int block_cols;
-  int idx32;
-  int small;       // little work per compute unit: four-wave tiles
-};
-
-// LINES block columns starting at `bj` (identical patterns when LINES > 1), output
-// rows [m0, m0 + Cfg::TM).  Only the first `lines` of the LINES columns exist; the others are
-// computed on the last one's blocks and dropped.
-template <class Cfg, int BLK, bool TRANS_B, bool FULL, int LINES>
-__device__ __forceinline__ void dds_tile(const DdsArgs& g, int bj, int m0, char* smem, int lines = LINES) {
-  static_assert(Cfg::TN == LINES * BLK && Cfg::B_PARTS == LINES && Cfg::B_KMAJOR == TRANS_B, "one operand part per block column");
-  constexpr int KT = Cfg::KT;
-  constexpr int kTilesPerBlock = BLK / KT;
-  int start[LINES];
-#pragma unroll
-  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bj + (l < lines ? l : lines - 1)];
-  const int nseg = g.walk_offsets[bj + 1] - start[0];
-  const elem_t* a0 = g.lhs + (int64_t)m0 * (Cfg::A_KMAJOR ? g.lda : 1);
-  const int64_t a_kstride = Cfg::A_KMAJOR ? 1 : g.lda;
-  const int64_t a_part = (int64_t)Cfg::PM * (Cfg::A_KMAJOR ? g.lda : 1);
-  const int m_valid = (g.m - m0 < Cfg::TM) ? g.m - m0 : Cfg::TM;
-  const int lane = threadIdx.x & 63;
-  f32x16_t acc[Cfg::IM][Cfg::JN] = {};
-  for (int s0 = 0; s0 < nseg; s0 += kMaxSegments) {
-    const int cnt = (nseg - s0 < kMaxSegments) ? nseg - s0 : kMaxSegments;
-    // Lane i of every wavefront holds the (k block, block id) pair of walk entry s0 + i, so
-    // that the K loop gets them with a lane read instead of a load.
-    const int e = lane < cnt ? lane : cnt - 1;
-    const int seg_k = load_index(g.walk_columns, start[0] + s0 + e, g.idx32);
-    int seg_block[LINES];
-#pragma unroll
-    for (int l = 0; l < LINES; l++) seg_block[l] = TRANS_B ? start[l] + s0 + e : g.walk_blocks[start[l] + s0 + e];
-    auto tile_fn = [&](int t) {
-      const int seg = t / kTilesPerBlock, sub = t % kTilesPerBlock;
-      const int64_t kb = __builtin_amdgcn_readlane(seg_k, seg);
-      TilePtrs p;
-      p.a[0] = a0 + (kb * BLK + sub * KT) * a_kstride;
-      p.a[1] = p.a[0] + a_part;
-#pragma unroll
-      for (int l = 0; l < LINES; l++)
-        p.b[l] = g.data + (int64_t)__builtin_amdgcn_readlane(seg_block[l], seg) * (BLK * BLK) + sub * KT * (TRANS_B ? 1 : BLK);
-      p.k_valid = KT;
-      return p;
-    };
-    if constexpr (FULL) mainloop_dma<Cfg>(acc, cnt * kTilesPerBlock, tile_fn, g.lda, BLK, smem);
-    else mainloop_reg<Cfg>(acc, cnt * kTilesPerBlock, tile_fn, g.lda, BLK, m_valid, BLK, smem);
-  }
-  const WaveCoords w = wave_coords<Cfg>();
-  const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + (int64_t)(m0 + wm0) * g.ldc + (int64_t)bj * BLK + wn0, g.ldc, m_valid - wm0, lines * BLK - wn0, smem);
-}
 
 // One block column per workgroup (four wavefronts).
 template <class Cfg, int BLK, bool TRANS_B, bool FULL>
@@ -155,11 +90,6 @@ __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists 
   }
 }
 
-template <class Kernel>
-static void set_lds_limit(Kernel kernel, int bytes) {
-  if (bytes > 60000) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 template <class Cfg, int BLK, bool TRANS_B, bool FULL>
 static void launch_one(const DdsArgs& g, hipStream_t stream) {
   static const int once = (set_lds_limit(&dds_kernel<Cfg, BLK, TRANS_B, FULL>, Cfg::kSmemBytes), 0);
@@ -214,32 +144,36 @@ static void launch_dds(const DdsArgs& g, const PlanLists& plan, hipStream_t stre
 
 }  // namespace stk
 
-extern "C" int stk_dds(int64_t m, int64_t k, int64_t n,
-                       const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
-                       const void* data, const int32_t* offsets, const void* column_indices,
-                       const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
-                       int transpose_b,
-                       void* out, int64_t out_stride_m,
-                       int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
-  using namespace stk;
-  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "stk_dds: blocking %d (64 or 128)", blocking);
-  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "stk_dds: dtype %d", dtype);
-  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_dds: index dtype %d", index_dtype);
-  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "stk_dds: negative size");
+// Checks the arguments of a dds and turns them into the kernels' view of the problem.  STK_OK with p->empty set when
+// there is nothing to compute.
+int stk::dds_problem(const char* who, int64_t m, int64_t k, int64_t n,
+                     const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                     const void* data, const int32_t* offsets, const void* column_indices,
+                     const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                     int transpose_b, void* out, int64_t out_stride_m,
+                     int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, DdsProblem* p) {
+  p->empty = false;
+  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "%s: blocking %d (64 or 128)", who, blocking);
+  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "%s: index dtype %d", who, index_dtype);
+  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "%s: negative size", who);
   if (k % blocking || n % blocking || m % 8)
     return fail(STK_ERR_DIMS, "incompatible dimensions: dense [%lld, %lld] x sparse [%lld, %lld] with blocking %d",
                 (long long)m, (long long)k, (long long)k, (long long)n, blocking);
-  if (m == 0 || n == 0) return STK_OK;
+  if (m == 0 || n == 0) {
+    p->empty = true;
+    return STK_OK;
+  }
   const int64_t block_cols = n / blocking;
-  if (block_cols * ((m + 63) / 64) > INT32_MAX || m > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "stk_dds: size exceeds 32-bit range");
+  if (block_cols * ((m + 63) / 64) > INT32_MAX || m > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "%s: size exceeds 32-bit range", who);
   const bool ak = lhs_stride_k == 1;   // row-major lhs: K-major tile
-  if (!ak && lhs_stride_m != 1) return fail(STK_ERR_UNSUPPORTED, "stk_dds: lhs needs a unit stride");
+  if (!ak && lhs_stride_m != 1) return fail(STK_ERR_UNSUPPORTED, "%s: lhs needs a unit stride", who);
   const int64_t lda = ak ? lhs_stride_m : lhs_stride_k;
   if (lda % 8 || out_stride_m % 8 || !aligned16(lhs) || !aligned16(out) || !aligned16(data))
-    return fail(STK_ERR_UNSUPPORTED, "stk_dds: operands need 16-byte aligned bases and leading dimensions divisible by 8");
-  if (lda >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "stk_dds: leading dimension exceeds 2^24 elements");
+    return fail(STK_ERR_UNSUPPORTED, "%s: operands need 16-byte aligned bases and leading dimensions divisible by 8", who);
+  if (lda >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "%s: leading dimension exceeds 2^24 elements", who);
   const bool tb = transpose_b != 0;
-  DdsArgs g;
+  DdsArgs& g = p->g;
   g.lhs = static_cast<const elem_t*>(lhs);
   g.lda = lda;
   g.data = static_cast<const elem_t*>(data);
@@ -254,13 +188,33 @@ extern "C" int stk_dds(int64_t m, int64_t k, int64_t n,
   // a dense-operand column panel (one block of k) is read once per tile that walks a block in that block row of
   // op(S): with few blocks per row it is streamed
   // (lhs with unit stride along m only: a K-major tile uses half a cache line per K-tile and needs the line to stay)
-  const bool stream_lhs = !ak && nnz <= 4 * (k / blocking);
+  p->stream_lhs = !ak && nnz <= 4 * (k / blocking);
+  p->ak = ak;
+  p->tb = tb;
   g.small = nnz * (m / 128) < kSmallWorkPerUnit * compute_units();
-  if (!g.walk_offsets || (nnz > 0 && (!g.walk_columns || (!tb && !g.walk_blocks) || !data))) return fail(STK_ERR_DIMS, "stk_dds: missing metadata pointer");
+  if (!g.walk_offsets || (nnz > 0 && (!g.walk_columns || (!tb && !g.walk_blocks) || !data))) return fail(STK_ERR_DIMS, "%s: missing metadata pointer", who);
   // lists of the walked lines: block columns of the stored matrix [k, n], or block rows of the stored [n, k]
-  PlanLists lists{nullptr, nullptr, 0};
-  if (plan) lists = tb ? plan_lists_of(plan_body(plan, n / blocking, nnz), n / blocking, k / blocking, false)
-                       : plan_lists_of(plan_body(plan, k / blocking, nnz), k / blocking, n / blocking, true);
+  p->lists = PlanLists{nullptr, nullptr, 0};
+  if (plan) p->lists = tb ? plan_lists_of(plan_body(plan, n / blocking, nnz), n / blocking, k / blocking, false)
+                          : plan_lists_of(plan_body(plan, k / blocking, nnz), k / blocking, n / blocking, true);
+  return STK_OK;
+}
+
+extern "C" int stk_dds(int64_t m, int64_t k, int64_t n,
+                       const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                       const void* data, const int32_t* offsets, const void* column_indices,
+                       const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                       int transpose_b,
+                       void* out, int64_t out_stride_m,
+                       int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
+  using namespace stk;
+  DdsProblem problem;
+  const int rc = dds_problem("stk_dds", m, k, n, lhs, lhs_stride_m, lhs_stride_k, data, offsets, column_indices, offsets_t, column_indices_t,
+                             block_offsets_t, transpose_b, out, out_stride_m, nnz, blocking, dtype, index_dtype, plan, &problem);
+  if (rc != STK_OK || problem.empty) return rc;
+  const DdsArgs& g = problem.g;
+  const PlanLists& lists = problem.lists;
+  const bool ak = problem.ak, tb = problem.tb, stream_lhs = problem.stream_lhs;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define STK_DDS_CASE(BF, BLK, AK, TB)                                         \
   if ((dtype == STK_BF16) == BF && blocking == BLK && ak == AK && tb == TB) { \

@@ -5,88 +5,9 @@
 // tile of the dense operand - for one tile of output columns.  It walks the nonzero blocks
 // of the row (for a transposed sparse operand: the CSC column segment with
 // indirect block ids).
-#include "common.h"
-#include "gemm_core.h"
+#include "dsd_tile.h"
 
 namespace stk {
-
-constexpr int kMaxSegments = 64;  // walk entries held at a time, one per lane of every wavefront
-
-struct DsdArgs {
-  const elem_t* data;
-  const int32_t* walk_offsets;
-  const void* walk_columns;
-  const int32_t* walk_blocks;  // indirect block ids (transposed operand) or null
-  const elem_t* rhs;
-  int64_t ldb;
-  elem_t* out;
-  int64_t ldc;
-  int block_rows;
-  int n;
-  int idx32;
-  int small;       // little work per compute unit: four-wave tiles
-};
-
-// acc += the products of walk entries [e0, e1) of LINES block rows starting at `bi` (identical
-// patterns when LINES > 1) with output columns [n0, n0 + Cfg::TN).  Only the first `lines` of the
-// LINES rows exist; the others are computed on the last one's blocks and dropped by the caller.
-template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES>
-__device__ __forceinline__ void dsd_accumulate(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, int e0, int e1, char* smem,
-                                               int lines = LINES) {
-  static_assert(Cfg::TM == LINES * BLK && Cfg::A_PARTS == LINES && Cfg::A_KMAJOR == !TRANS_A, "one operand part per block row");
-  constexpr int KT = Cfg::KT;
-  constexpr int kTilesPerBlock = BLK / KT;
-  int start[LINES];
-#pragma unroll
-  for (int l = 0; l < LINES; l++) start[l] = g.walk_offsets[bi + (l < lines ? l : lines - 1)];
-  const elem_t* b0 = g.rhs + (int64_t)n0 * (Cfg::B_KMAJOR ? g.ldb : 1);
-  const int64_t b_kstride = Cfg::B_KMAJOR ? 1 : g.ldb;
-  const int64_t b_part = (int64_t)Cfg::PN * (Cfg::B_KMAJOR ? g.ldb : 1);
-  const int n_valid = (g.n - n0 < Cfg::TN) ? g.n - n0 : Cfg::TN;
-  const int lane = threadIdx.x & 63;
-  for (int s0 = e0; s0 < e1; s0 += kMaxSegments) {
-    const int cnt = (e1 - s0 < kMaxSegments) ? e1 - s0 : kMaxSegments;
-    // Lane i of every wavefront holds the (k block, block id) pair of walk entry s0 + i, so
-    // that the K loop gets them with a lane read instead of a load.
-    const int e = lane < cnt ? lane : cnt - 1;
-    const int seg_k = load_index(g.walk_columns, start[0] + s0 + e, g.idx32);
-    int seg_block[LINES];
-#pragma unroll
-    for (int l = 0; l < LINES; l++) seg_block[l] = TRANS_A ? g.walk_blocks[start[l] + s0 + e] : start[l] + s0 + e;
-    auto tile_fn = [&](int t) {
-      const int seg = t / kTilesPerBlock, sub = t % kTilesPerBlock;
-      const int64_t kb = __builtin_amdgcn_readlane(seg_k, seg);
-      TilePtrs p;
-#pragma unroll
-      for (int l = 0; l < LINES; l++)
-        p.a[l] = g.data + (int64_t)__builtin_amdgcn_readlane(seg_block[l], seg) * (BLK * BLK) + sub * KT * (TRANS_A ? BLK : 1);
-      p.b[0] = b0 + (kb * BLK + sub * KT) * b_kstride;
-      p.b[1] = p.b[0] + b_part;
-      p.k_valid = KT;
-      return p;
-    };
-    if constexpr (FULL) mainloop_dma<Cfg>(acc, cnt * kTilesPerBlock, tile_fn, BLK, g.ldb, smem);
-    else mainloop_reg<Cfg>(acc, cnt * kTilesPerBlock, tile_fn, BLK, g.ldb, BLK, n_valid, smem);
-  }
-}
-
-// Writes the finished tile: the first `rows` rows from block row `bi` onwards, columns from n0.
-template <class Cfg, int BLK>
-__device__ __forceinline__ void dsd_store(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, char* smem, int rows = Cfg::TM) {
-  const int n_valid = (g.n - n0 < Cfg::TN) ? g.n - n0 : Cfg::TN;
-  const WaveCoords w = wave_coords<Cfg>();
-  const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, rows - wm0, n_valid - wn0, smem);
-}
-
-// The whole tile of LINES block rows starting at `bi` (the first `lines` of them exist), output columns
-// [n0, n0 + Cfg::TN).
-template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES>
-__device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char* smem, int lines = LINES) {
-  f32x16_t acc[Cfg::IM][Cfg::JN] = {};
-  dsd_accumulate<Cfg, BLK, TRANS_A, FULL, LINES>(acc, g, bi, n0, 0, g.walk_offsets[bi + 1] - g.walk_offsets[bi], smem, lines);
-  dsd_store<Cfg, BLK>(acc, g, bi, n0, smem, lines * BLK);
-}
 
 // One block row per workgroup (four wavefronts).
 template <class Cfg, int BLK, bool TRANS_A, bool FULL>
@@ -355,11 +276,6 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   dsd_slice<Single, TRANS_A, 1>(g, t, const_ints(plan.list(kTallSingles))[i / ntn], (i % ntn) * Single::TN, slice, slices, ordinal, smem, &flag);
 }
 
-template <class Kernel>
-static void set_lds_limit(Kernel kernel, int bytes) {
-  if (bytes > 60000) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 template <class Cfg, int BLK, bool TRANS_A, bool FULL>
 static void launch_one(const DsdArgs& g, hipStream_t stream) {
   static const int once = (set_lds_limit(&dsd_kernel<Cfg, BLK, TRANS_A, FULL>, Cfg::kSmemBytes), 0);
@@ -431,33 +347,36 @@ static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* 
 
 }  // namespace stk
 
-extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
-                       const void* data, const int32_t* offsets, const void* column_indices,
-                       const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
-                       int transpose_a,
-                       const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
-                       void* out, int64_t out_stride_m,
-                       int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
-                       void* workspace, int64_t workspace_bytes, stk_stream_t stream) {
-  using namespace stk;
-  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: blocking %d (64 or 128)", blocking);
-  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: dtype %d", dtype);
-  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: index dtype %d", index_dtype);
-  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "stk_dsd: negative size");
+// Checks the arguments of a dsd and turns them into the kernels' view of the problem.  STK_OK with p->empty set when
+// there is nothing to compute.
+int stk::dsd_problem(const char* who, int64_t m, int64_t k, int64_t n,
+                     const void* data, const int32_t* offsets, const void* column_indices,
+                     const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                     int transpose_a, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                     void* out, int64_t out_stride_m, int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                     DsdProblem* p) {
+  p->empty = false;
+  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "%s: blocking %d (64 or 128)", who, blocking);
+  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "%s: index dtype %d", who, index_dtype);
+  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "%s: negative size", who);
   if (m % blocking || k % blocking || n % 8)
     return fail(STK_ERR_DIMS, "incompatible dimensions: sparse [%lld, %lld] x dense [%lld, %lld] with blocking %d",
                 (long long)m, (long long)k, (long long)k, (long long)n, blocking);
-  if (m == 0 || n == 0) return STK_OK;
+  if (m == 0 || n == 0) {
+    p->empty = true;
+    return STK_OK;
+  }
   const int64_t block_rows = m / blocking;
-  if (block_rows * ((n + 63) / 64) > INT32_MAX || n > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: size exceeds 32-bit range");
+  if (block_rows * ((n + 63) / 64) > INT32_MAX || n > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "%s: size exceeds 32-bit range", who);
   const bool bk = rhs_stride_n != 1;   // .t() view of a row-major [n, k]: K-major tile
-  if (bk && rhs_stride_k != 1) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: rhs needs a unit stride");
+  if (bk && rhs_stride_k != 1) return fail(STK_ERR_UNSUPPORTED, "%s: rhs needs a unit stride", who);
   const int64_t ldb = bk ? rhs_stride_n : rhs_stride_k;
   if (ldb % 8 || out_stride_m % 8 || !aligned16(rhs) || !aligned16(out) || !aligned16(data))
-    return fail(STK_ERR_UNSUPPORTED, "stk_dsd: operands need 16-byte aligned bases and leading dimensions divisible by 8");
-  if (ldb >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "stk_dsd: leading dimension exceeds 2^24 elements");
+    return fail(STK_ERR_UNSUPPORTED, "%s: operands need 16-byte aligned bases and leading dimensions divisible by 8", who);
+  if (ldb >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "%s: leading dimension exceeds 2^24 elements", who);
   const bool ta = transpose_a != 0;
-  DsdArgs g;
+  DsdArgs& g = p->g;
   g.data = static_cast<const elem_t*>(data);
   g.walk_offsets = ta ? offsets_t : offsets;
   g.walk_columns = ta ? column_indices_t : column_indices;
@@ -472,13 +391,35 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
   // a dense-operand row panel (one block of k) is read once per tile that walks a block in that block column of
   // op(S): with few blocks per column (a block-diagonal MoE layout has one fused tile per expert) it is streamed
   // (row-major rhs only: a K-major tile uses half a cache line per K-tile and needs the line to stay)
-  const bool stream_rhs = !bk && nnz <= 4 * (k / blocking);
+  p->stream_rhs = !bk && nnz <= 4 * (k / blocking);
+  p->ta = ta;
+  p->bk = bk;
   g.small = nnz * (n / 128) < kSmallWorkPerUnit * compute_units();
-  if (!g.walk_offsets || (nnz > 0 && (!g.walk_columns || (ta && !g.walk_blocks) || !data))) return fail(STK_ERR_DIMS, "stk_dsd: missing metadata pointer");
+  if (!g.walk_offsets || (nnz > 0 && (!g.walk_columns || (ta && !g.walk_blocks) || !data))) return fail(STK_ERR_DIMS, "%s: missing metadata pointer", who);
   // lists of the walked lines: block rows of the stored matrix [m, k], or block columns of the stored [k, m]
-  PlanLists lists{nullptr, nullptr, 0};
-  if (plan) lists = ta ? plan_lists_of(plan_body(plan, k / blocking, nnz), k / blocking, m / blocking, true)
-                       : plan_lists_of(plan_body(plan, m / blocking, nnz), m / blocking, k / blocking, false);
+  p->lists = PlanLists{nullptr, nullptr, 0};
+  if (plan) p->lists = ta ? plan_lists_of(plan_body(plan, k / blocking, nnz), k / blocking, m / blocking, true)
+                          : plan_lists_of(plan_body(plan, m / blocking, nnz), m / blocking, k / blocking, false);
+  return STK_OK;
+}
+
+extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
+                       const void* data, const int32_t* offsets, const void* column_indices,
+                       const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                       int transpose_a,
+                       const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                       void* out, int64_t out_stride_m,
+                       int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                       void* workspace, int64_t workspace_bytes, stk_stream_t stream) {
+  using namespace stk;
+  DsdProblem problem;
+  const int rc = dsd_problem("stk_dsd", m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, transpose_a, rhs,
+                             rhs_stride_k, rhs_stride_n, out, out_stride_m, nnz, blocking, dtype, index_dtype, plan, &problem);
+  if (rc != STK_OK || problem.empty) return rc;
+  const DsdArgs& g = problem.g;
+  const PlanLists& lists = problem.lists;
+  const bool ta = problem.ta, bk = problem.bk, stream_rhs = problem.stream_rhs;
+  const int64_t block_rows = g.block_rows;
   // Sliced last round: for launches of a few rounds of tiles (with many rounds the last one matters little and
   // the plain kernel is used as it is); the plan says whether and how the last round is cut.
   TailArgs tail{};

@@ -294,6 +294,8 @@ struct TileCfg {
   static constexpr int kAccRegs = IM * JN;
 };
 
+constexpr int kMaxSegments = 64;  // walk entries of a sparse line held at a time, one per lane of every wavefront
+
 struct TilePtrs {
   const elem_t* a[4];  // element (m = 0, k = 0) of each part of the A tile
   const elem_t* b[4];  // element (k = 0, n = 0) of each part of the B tile

@@ -197,11 +197,6 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void sdd_single_kernel(SddArgs g)
   sdd_tile<Cfg, BLK, FULL>(g, rr, cc, pp, smem);
 }
 
-template <class Kernel>
-static void set_lds_limit(Kernel kernel, int bytes) {
-  if (bytes > 60000) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 // 128-blocks with k a multiple of the K-tile depth KT: the direct-to-LDS pipeline with STAGES ring stages.
 template <bool BF16, bool AK, bool BK, bool STREAM, int KT, int STAGES>
 static void launch_sdd128(const SddArgs& g, hipStream_t stream) {

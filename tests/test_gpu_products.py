@@ -486,6 +486,37 @@ def test_results_do_not_depend_on_the_fusion_plan(monkeypatch, b):
     U.assert_close(plain[1], O.dsd(topo.shape, U.np32(h0.data), topo, False, U.np32(w2)), dtype, "dsd without plan")
 
 
+@pytest.mark.parametrize("dtype,blocking,hidden", [(torch.bfloat16, 128, 1024), (torch.float16, 128, 512), (torch.bfloat16, 128, 256),
+                                                   (torch.float16, 64, 1024)])
+def test_both_gradients_of_sdd_in_one_call(dtype, blocking, hidden, monkeypatch):
+    # stk_dsd_dds: dS rhs^T and lhs^T dS from one call (one launch for 128-blocks with enough work; otherwise the two
+    # products one after the other) against the oracle's dsd and dds, and bit for bit against the separate launches
+    from stk_amd.backend import autograd, hip_kernels
+    monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
+    tokens = np.array([300, 0, 129, 384, 640, 128, 77, 256, 512, 1000, 40, 896])
+    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden, 2048, blocking, dtype, 31)
+    g = torch.Generator().manual_seed(32)
+    ds = (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV)
+    dsm = stk.Matrix(tm.size(), ds, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
+    rows, cols = tm.size()
+    dx = torch.full((rows, hidden), float("nan"), dtype=dtype, device=DEV)
+    dw1 = torch.full((hidden, cols), float("nan"), dtype=dtype, device=DEV)
+    hip_kernels.dsd_dds(tm.size(), ds, tm.offsets, tm.row_indices, tm.column_indices, tm.offsets_t, tm.column_indices_t, tm.block_offsets_t,
+                        w1.t(), dx, x.t(), dw1)
+    U.assert_close(dx, O.dsd(topo.shape, U.np32(ds), topo, False, U.np32(w1).T), dtype, "dS W1^T")
+    U.assert_close(dw1, O.dds(U.np32(x).T, topo.shape, U.np32(ds), topo, False), dtype, "x^T dS")
+    assert torch.equal(dx, stk.ops.dsd(dsm, w1.t())) and torch.equal(dw1, stk.ops.dds(x.t(), dsm))
+    # through autograd: the gradients of sdd with the joint call and with two launches
+    grads = {}
+    for joint in (True, False):
+        monkeypatch.setattr(autograd, "JOINT_GRADIENTS", joint)
+        xs, ws = x.detach().clone().requires_grad_(True), w1.detach().clone().requires_grad_(True)
+        stk.ops.sdd(xs, ws, tm).data.backward(ds)
+        grads[joint] = (xs.grad, ws.grad)
+    assert torch.equal(grads[True][0], grads[False][0]) and torch.equal(grads[True][1], grads[False][1])
+    assert torch.equal(grads[True][0], dx) and torch.equal(grads[True][1], dw1)
+
+
 def test_gradients_side_by_side_equal_gradients_one_after_the_other(monkeypatch):
     # backward launches the two gradients of a product on two streams; same kernels, so the same bits
     from stk_amd.backend import autograd
