@@ -345,21 +345,63 @@ __global__ __launch_bounds__(256) void block_mask_kernel(const E* __restrict__ x
   }
 }
 
-// offsets[0] = 0, offsets[r + 1] = number of nonzero blocks in rows 0..r.  One workgroup.
+// The same with 16 bytes per lane, for blocks whose rows are a power-of-two number (at most 64) of aligned
+// 16-byte pieces: a wavefront covers 64 >> log2_pieces block rows per load and keeps four loads in flight.
+template <int ELEM_BYTES>
+__global__ __launch_bounds__(256) void block_mask_vec_kernel(const char* __restrict__ x, int64_t ld_bytes, int b, int log2_pieces,
+                                                             int block_cols, int64_t blocks, uint8_t* __restrict__ mask) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave0 = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) >> 6;
+  const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  constexpr uint32_t kAbs = ELEM_BYTES == 2 ? 0x7fff7fffu : 0x7fffffffu;   // everything but the sign bits
+  const int rows_per_load = 64 >> log2_pieces;
+  const int row0 = lane >> log2_pieces;
+  const int64_t lane_offset = (int64_t)row0 * ld_bytes + (int64_t)(lane & ((1 << log2_pieces) - 1)) * 16;
+  for (int64_t blk = wave0; blk < blocks; blk += nwaves) {
+    const int64_t r = blk / block_cols, c = blk - r * block_cols;
+    const char* base = x + r * b * ld_bytes + c * (int64_t)b * ELEM_BYTES + lane_offset;
+    uint32_t any = 0;
+    for (int i0 = 0; i0 < b; i0 += 4 * rows_per_load) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int i = i0 + u * rows_per_load + row0;
+        v[u] = make_uint4(0u, 0u, 0u, 0u);
+        if (i < b) v[u] = *reinterpret_cast<const uint4*>(base + (int64_t)(i0 + u * rows_per_load) * ld_bytes);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) any |= (v[u].x | v[u].y | v[u].z | v[u].w) & kAbs;
+    }
+    const uint64_t bal = __ballot(any != 0);
+    if (lane == 0) mask[blk] = bal != 0;
+  }
+}
+
+// offsets[0] = 0, offsets[r + 1] = number of nonzero blocks in rows 0..r.  One workgroup; a wavefront counts a
+// block row at a time (coalesced reads of the mask), sixteen rows per round, then a scan over the rounds' counts.
 __global__ __launch_bounds__(1024) void row_offsets_kernel(const uint8_t* __restrict__ mask, int block_rows, int block_cols,
                                                            int32_t* __restrict__ offsets) {
   __shared__ int part[16];
+  __shared__ int counts[1024];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int carry = 0;
   if (threadIdx.x == 0) offsets[0] = 0;
   for (int r0 = 0; r0 < block_rows; r0 += 1024) {
-    int r = r0 + threadIdx.x;
-    int cnt = 0;
-    if (r < block_rows)
-      for (int c = 0; c < block_cols; c++) cnt += mask[(int64_t)r * block_cols + c];
+    // rows r0 + wave, r0 + wave + 16, ...: one per wavefront and step
+    for (int q = wave; q < 1024 && r0 + q < block_rows; q += 16) {
+      int cnt = 0;
+      for (int c = lane; c < block_cols; c += kWave) cnt += mask[(int64_t)(r0 + q) * block_cols + c];
+      cnt = wave_inclusive_scan(cnt, lane);
+      if (lane == kWave - 1) counts[q] = cnt;
+    }
+    __syncthreads();
+    const int r = r0 + threadIdx.x;
+    const int cnt = r < block_rows ? counts[threadIdx.x] : 0;
     int total;
-    int ex = block_exclusive_scan(cnt, part, &total);
+    const int ex = block_exclusive_scan(cnt, part, &total);
     if (r < block_rows) offsets[r + 1] = carry + ex + cnt;
     carry += total;
+    __syncthreads();
   }
 }
 
@@ -516,7 +558,21 @@ extern "C" int stk_to_sparse_count(const void* x, int64_t rows, int64_t cols, in
   if (br > INT32_MAX || bc > INT32_MAX || (int64_t)blocking * blocking > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_count: size exceeds 32-bit range");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t blocks = br * bc;
-  if (blocks > 0) {
+  // 16-byte loads when a block row is a power-of-two number (up to 64) of aligned 16-byte pieces
+  const int64_t row_bytes = (int64_t)blocking * elem_bytes;
+  int log2_pieces = -1;
+  if (row_bytes % 16 == 0 && (x_stride * elem_bytes) % 16 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0)
+    for (int l = 0; l <= 6; l++)
+      if (row_bytes == (16 << l)) log2_pieces = l;
+  if (blocks > 0 && log2_pieces >= 0) {
+    const int grid = (int)((blocks + 3) / 4 < 262144 ? (blocks + 3) / 4 : 262144);
+    if (elem_bytes == 2)
+      hipLaunchKernelGGL((block_mask_vec_kernel<2>), dim3(grid), dim3(256), 0, s, static_cast<const char*>(x), x_stride * elem_bytes, blocking,
+                         log2_pieces, (int)bc, blocks, mask);
+    else
+      hipLaunchKernelGGL((block_mask_vec_kernel<4>), dim3(grid), dim3(256), 0, s, static_cast<const char*>(x), x_stride * elem_bytes, blocking,
+                         log2_pieces, (int)bc, blocks, mask);
+  } else if (blocks > 0) {
     const int grid = (int)((blocks + 3) / 4 < 65536 ? (blocks + 3) / 4 : 65536);
     if (elem_bytes == 2)
       hipLaunchKernelGGL((block_mask_kernel<uint16_t>), dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(x), x_stride, blocking, (int)bc, blocks, mask);
