@@ -26,7 +26,8 @@
 //
 // A plan built for blocking 64 groups the lines by fours instead (stk_dsd and stk_dds then compute up to four
 // identical lines as one 256-wide tile): a run of identical lines is cut from its start into fours while they
-// last, and the three, two or one lines that are left form one more group.  Lines so long that a tile over four
+// last, and the three, two or one lines that are left form one more group (a four and one line left over become
+// a three and a pair).  Lines so long that a tile over four
 // of them would be more than a compute unit's share of the whole product (four times their blocks exceed
 // 4 nnz / compute units: the expert that takes half of the tokens of a skewed routing) are cut into pairs
 // instead, which the kernels start first.  Both role arrays then hold, for the
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(256) void plan_same_kernel(
 // Block rows of the sdd tile that line i owns (0: an earlier line's tile covers it).  pos: its place in its run
 // of identical lines.  same[j]: line j + 1 repeats line j (0 for the last line).
 //   most == 4: the run is cut from its start into fours while they last; what is left - three, two or one
-//              lines - forms one more group;
+//              lines - forms one more group (a four and one line left over become a three and a pair);
 //   most == 2: into pairs, and the last three lines of a run of odd length (three or more) form a group of
 //              three, whose tiles are one block wide; a run of one line is a single line.
 __device__ __forceinline__ int sdd_rows_owned(const uint8_t* same, int i, int pos, int most) {
@@ -161,11 +162,19 @@ __device__ __forceinline__ int sdd_rows_owned(const uint8_t* same, int i, int po
     if (left == 1) return pos == 0 ? 1 : 0;  // the third line of a group of three
     return 2;
   }
-  const int q = pos & 3, g = i - q;
-  int left = 1;  // lines from the group's first line to the end of the run, at most four
-  while (left < 4 && same[g + left - 1]) left++;
-  if (left >= 3) return q == 0 ? left : 0;  // (three lines: one tile of four whose last row is dropped)
-  if (q == 0) return left;                  // a pair or a single line
+  // most == 4.  A run of n lines is cut from its start into fours; what is left forms one more group of three or
+  // two, or a lone line if the run is one line - except that the last five lines of a run of 4 q + 1 lines (q >= 1)
+  // form a three and a pair rather than a four and a lone line, which would run on a tile with most of its rows
+  // dropped.  Seen from a line: groups start at positions 0, 4, 8, ... and, for that pair, at the position 3 mod 4
+  // from which exactly two lines are left.
+  const int q = pos & 3;
+  int left = 1;  // lines from this one to the end of the run, at most six
+  while (left < 6 && same[i + left - 1]) left++;
+  if (q == 0) {
+    if (left == 1 && pos >= 4) return 0;  // the last line of a run of 4 q + 1: covered by the pair before it
+    return left >= 6 || left == 4 ? 4 : (left == 5 ? 3 : left);
+  }
+  if (q == 3 && left == 2) return 2;
   return 0;
 }
 // The same for the groups of stk_dsd / stk_dds with 64-blocks: fours (as above) unless the lines are `heavy`, then

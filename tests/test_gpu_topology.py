@@ -292,11 +292,26 @@ def _groups_of_up_to_four(offsets, indices):
         n = 1
         while i + n < lines and len(seg[i]) > 0 and seg[i + n] == seg[i]:
             n += 1
-        most = 2 if 4 * len(seg[i]) > share else 4
-        for a in range(0, n, most):
-            size[i + a] = min(most, n - a)
+        if 4 * len(seg[i]) > share:
+            for a in range(0, n, 2):
+                size[i + a] = min(2, n - a)
+        else:
+            for a, r in _fours(n):
+                size[i + a] = r
         i += n
     return size
+
+
+def _fours(n):
+    """(first line, lines) of the groups a run of n identical lines is cut into: fours from the start, then the
+    three, two or one lines left - but a four and one line left over become a three and a pair."""
+    groups, a = [], 0
+    while a < n:
+        left = n - a
+        r = 4 if left >= 6 or left == 4 else (3 if left == 5 else left)
+        groups.append((a, r))
+        a += r
+    return groups
 
 
 def _sdd_tiles(offsets, indices, most_rows, most_cols):
@@ -317,7 +332,7 @@ def _sdd_tiles(offsets, indices, most_rows, most_cols):
         a = 0
         while a < n:
             if most_rows == 4:
-                r = min(4, n - a)
+                r = dict(_fours(n))[a]
             else:
                 r = 3 if n - a == 3 else min(2, n - a)
             wide = 1 if (r == 3 and most_cols == 2) else most_cols
