@@ -268,6 +268,33 @@ def routing_times(dev, steps, warmup, seed=0):
     return out
 
 
+def gradient_pair_times(topo, x, w1, calls):
+    """The two operand gradients of sdd on the benchmark topology, dsd(dS, W1^T) and dds(x^T, dS), as the one launch of
+    stk_dsd_dds and as two launches (stk_dsd without its workspace, stk_dds); `calls` times each, back to back."""
+    from stk_amd.backend import hip_kernels
+    ds = torch.empty_like(topo.data).normal_(0, 0.02)
+    meta = (topo.offsets, topo.row_indices, topo.column_indices, topo.offsets_t, topo.column_indices_t, topo.block_offsets_t)
+    dx, dw1 = torch.empty_like(x), torch.empty_like(w1)
+    slicing, hip_kernels.SLICE_LAST_ROUND = hip_kernels.SLICE_LAST_ROUND, False
+
+    def joint():
+        hip_kernels.dsd_dds(topo.size(), ds, *meta, w1.t(), dx, x.t(), dw1)
+
+    def two():
+        hip_kernels.dsd(topo.size(), ds, *meta, False, w1.t(), dx)
+        hip_kernels.dds(x.t(), topo.size(), ds, *meta, False, dw1)
+
+    try:
+        for fn in (joint, two):
+            for _ in range(3):
+                fn()
+        out = {"joint_launch_ms": time_batch(joint, calls), "two_launches_ms": time_batch(two, calls)}
+    finally:
+        hip_kernels.SLICE_LAST_ROUND = slicing
+    out["note"] = "dsd(dS,W1^T) + dds(x^T,dS): stk_dsd_dds against stk_dsd (no workspace) followed by stk_dds, back to back"
+    return out
+
+
 def _expert_choices(name, seed=0):
     """[tokens, top_k] int32 expert choices of the dMoE configurations of BASELINE.json."""
     g = torch.Generator().manual_seed(seed)
@@ -399,6 +426,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB -> 1 GiB elementwise kernel (torch.neg), the known-size reference for the HBM counters")
+    ap.add_argument("--gradient-pair-only", action="store_true",
+                    help="run only the two operand gradients of sdd, as one launch and as two (for the counter profiles)")
     ap.add_argument("--configs", default="2,4,5,5skew",
                     help="comma-separated other configurations of BASELINE.json to time as well (2, 4, 5, 5skew); 'none' leaves them out")
     args = ap.parse_args()
@@ -421,6 +450,11 @@ def main():
     rows = topo.size()[0]
     xt = x.t()
     flops_op = nnz * 2.0 * BLOCK * BLOCK * HIDDEN
+
+    if args.gradient_pair_only:
+        with torch.no_grad():
+            print(json.dumps({"sdd_gradient_pair": gradient_pair_times(topo, x, w1, max(args.steps, 1))}))
+        return
 
     names = ("sdd", "dsd", "dds")
     state = {}
@@ -493,6 +527,7 @@ def main():
         per_op_ms = {n: float(np.mean([e[i].elapsed_time(e[i + 1]) for e in evs])) for i, n in enumerate(names)}
         # and each product on its own, back to back
         per_op_b2b_ms = {n: time_batch(product, args.steps) for n, product in zip(names, products)}
+        gradient_pair = gradient_pair_times(topo, x, w1, args.steps)
         gc.enable()
 
         others = {}
@@ -547,6 +582,7 @@ def main():
         "frac_of_dense_step": value / dense_step_tflops,
         "roofline": roof,
         "routing": routing,
+        "sdd_gradient_pair": gradient_pair,
     }
     if others:
         result["other_configs"] = others

@@ -41,7 +41,13 @@ extern "C" {
 #define STK_ERR_HIP 3         /* a HIP runtime call failed; see stk_last_error() */
 #define STK_ERR_WORKSPACE 4   /* workspace pointer missing or too small */
 
-/* element types of values */
+/*
+ * Element types of values.  The reference's launchers take whatever dtype the tensors have
+ * (stk/backend/triton_kernels.py:250, 306, 358 pass the pointers on, float32 included); the products here compute
+ * on 16-bit MFMA operands with fp32 accumulation and accept float16 and bfloat16 only.  Anything else is refused with
+ * STK_ERR_UNSUPPORTED - nothing is converted silently: a float32 caller rounds its operands to one of the two types
+ * itself and so chooses the precision it loses.  The format helpers (to_dense, to_sparse) take 2- and 4-byte elements.
+ */
 #define STK_F16 0
 #define STK_BF16 1
 
