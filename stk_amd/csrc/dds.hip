@@ -18,6 +18,22 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dds_kernel(DdsArgs g) {
   dds_tile<Cfg, BLK, TRANS_B, FULL, 1>(g, item / ntm, (item % ntm) * Cfg::TM, smem);
 }
 
+// Every block column on its own (four wavefronts), in the order of the plan's lists: the columns of the pairs,
+// then the lone columns longest first - for launches with little work per compute unit, where the order in which
+// the tiles start decides how evenly the units are loaded.
+template <class Cfg, int BLK, bool TRANS_B>
+__global__ __launch_bounds__(Cfg::kThreads, 2) void dds_lines_kernel(DdsArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  const int ntm = (g.m + Cfg::TM - 1) / Cfg::TM;
+  const int pairs = const_ints(plan.counts)[kPairs];
+  const int tiles = (2 * pairs + const_ints(plan.counts)[kSingles]) * ntm;
+  if ((int)blockIdx.x >= tiles) return;
+  const int item = xcd_grouped(blockIdx.x, tiles);
+  const int l = item / ntm;
+  const int line = l < 2 * pairs ? const_ints(plan.list(kPairs))[l >> 1] + (l & 1) : const_ints(plan.list(kSingles))[l - 2 * pairs];
+  dds_tile<Cfg, BLK, TRANS_B, true, 1>(g, line, (item % ntm) * Cfg::TM, smem);
+}
+
 // The lone block columns of a plan's list, one per workgroup (four wavefronts): what dds_fused64_kernel leaves.
 template <class Cfg, int BLK, bool TRANS_B, bool FULL>
 __global__ __launch_bounds__(Cfg::kThreads, 2) void dds_singles_kernel(DdsArgs g, PlanLists plan) {
@@ -85,7 +101,7 @@ __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists 
   }
   bid -= pair_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_item(bid, single_tiles, spread);
+    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
     dds_tile<Single, 128, TRANS_B, true, 1>(g, const_ints(plan.list(kSingles))[item / ntm], (item % ntm) * Single::TM, smem);
   }
 }
@@ -116,6 +132,11 @@ static void launch_dds(const DdsArgs& g, const PlanLists& plan, hipStream_t stre
       static const int once = (set_lds_limit(&dds_fused_kernel<Fused, Single, TRANS_B>, lds), 0);
       (void)once;
       hipLaunchKernelGGL((dds_fused_kernel<Fused, Single, TRANS_B>), dim3(g.block_cols * (g.m / Fused::TM)), dim3(512), lds, stream, g, plan);
+    } else if (g.m % Narrow::TM == 0 && plan.counts) {
+      static const int once = (set_lds_limit(&dds_lines_kernel<Narrow, BLK, TRANS_B>, Narrow::kSmemBytes), 0);
+      (void)once;
+      hipLaunchKernelGGL((dds_lines_kernel<Narrow, BLK, TRANS_B>), dim3(g.block_cols * (g.m / Narrow::TM)), dim3(Narrow::kThreads),
+                         Narrow::kSmemBytes, stream, g, plan);
     } else if (g.m % Narrow::TM == 0) {
       launch_one<Narrow, BLK, TRANS_B, true>(g, stream);
     } else {

@@ -18,6 +18,24 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_kernel(DsdArgs g) {
   dsd_tile<Cfg, BLK, TRANS_A, FULL, 1>(g, item / ntn, (item % ntn) * Cfg::TN, smem);
 }
 
+// Every block row on its own (four wavefronts), in the order of the plan's lists: the rows of the pairs, of the
+// threes, then the lone rows longest first - for launches with little work per compute unit, where the order in
+// which the tiles start decides how evenly the units are loaded.
+template <class Cfg, int BLK, bool TRANS_A>
+__global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_lines_kernel(DsdArgs g, PlanLists plan) {
+  extern __shared__ __align__(16) char smem[];
+  const int ntn = (g.n + Cfg::TN - 1) / Cfg::TN;
+  const int pairs = const_ints(plan.counts)[kTallPairs], triples = const_ints(plan.counts)[kTallTriples];
+  const int tiles = (2 * pairs + 3 * triples + const_ints(plan.counts)[kTallSingles]) * ntn;
+  if ((int)blockIdx.x >= tiles) return;
+  const int item = xcd_grouped(blockIdx.x, tiles);
+  int l = item / ntn, line;
+  if (l < 2 * pairs) line = const_ints(plan.list(kTallPairs))[l >> 1] + (l & 1);
+  else if ((l -= 2 * pairs) < 3 * triples) line = const_ints(plan.list(kTallTriples))[l / 3] + l % 3;
+  else line = const_ints(plan.list(kTallSingles))[l - 3 * triples];
+  dsd_tile<Cfg, BLK, TRANS_A, true, 1>(g, line, (item % ntn) * Cfg::TN, smem);
+}
+
 // The lone block rows of a plan's list, one per workgroup (four wavefronts): what dsd_fused64_kernel leaves.
 template <class Cfg, int BLK, bool TRANS_A, bool FULL>
 __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_singles_kernel(DsdArgs g, PlanLists plan) {
@@ -97,7 +115,7 @@ __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists 
   }
   bid -= triple_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_item(bid, single_tiles, spread);
+    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
     dsd_tile<Single, 128, TRANS_A, true, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
   }
 }
@@ -272,7 +290,7 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
     return;
   }
   item -= triple_tiles;
-  const int i = xcd_item(item, single_tiles, spread);
+  const int i = xcd_grouped(item, single_tiles);  // (in order of length: no contiguous shares)
   dsd_slice<Single, TRANS_A, 1>(g, t, const_ints(plan.list(kTallSingles))[i / ntn], (i % ntn) * Single::TN, slice, slices, ordinal, smem, &flag);
 }
 
@@ -319,6 +337,11 @@ static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* 
       static const int once = (set_lds_limit(&dsd_fused_kernel<Fused, Triple, Single, TRANS_A>, lds), 0);
       (void)once;
       hipLaunchKernelGGL((dsd_fused_kernel<Fused, Triple, Single, TRANS_A>), dim3(g.block_rows * (g.n / Fused::TN)), dim3(512), lds, stream, g, plan);
+    } else if (g.n % Narrow::TN == 0 && plan.counts) {
+      static const int once = (set_lds_limit(&dsd_lines_kernel<Narrow, BLK, TRANS_A>, Narrow::kSmemBytes), 0);
+      (void)once;
+      hipLaunchKernelGGL((dsd_lines_kernel<Narrow, BLK, TRANS_A>), dim3(g.block_rows * (g.n / Narrow::TN)), dim3(Narrow::kThreads),
+                         Narrow::kSmemBytes, stream, g, plan);
     } else if (g.n % Narrow::TN == 0) {
       launch_one<Narrow, BLK, TRANS_A, true>(g, stream);
     } else {

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
     }
     bid -= triple_tiles;
     if (bid < single_tiles) {
-      const int item = xcd_item(bid, single_tiles, spread);
+      const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
       dsd_tile<DsdSingle, 128, false, true, 1>(d, const_ints(rows.list(kTallSingles))[item / ntn], (item % ntn) * DsdSingle::TN, smem);
       return;
     }
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
   }
   bid -= pair_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_item(bid, single_tiles, spread);
+    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
     dds_tile<DdsSingle, 128, false, true, 1>(s, const_ints(cols.list(kSingles))[item / ntm], (item % ntm) * DdsSingle::TM, smem);
   }
 }

@@ -15,8 +15,10 @@
 //   tall[i] = 3  line i is computed together with lines i + 1 and i + 2
 // (0, 1, 2 as above).  A dense operand that is streamed once per tile is then read
 // once, not twice, for such a run of three.
-// Behind the roles come, as int32, ten counts and ten ascending lists of lines, five per
-// direction (block rows first): role 1, role 0, tall 1, tall 3, tall 0.  The product
+// Behind the roles come, as int32, ten counts and ten lists of lines, five per
+// direction (block rows first): role 1, role 0, tall 1, tall 3, tall 0 - ascending, except that the two lists of
+// lone lines (role 0, tall 0) are in order of descending length (min(blocks, 255); equal lengths ascending) when
+// they have at most 4096 entries.  The product
 // kernels take their work from these lists, so that no workgroup is launched for a
 // covered line.  Last come, per direction, sixteen bytes for stk_dsd: into how many slices
 // along k the tiles of the last, partly filled round of workgroups are cut when the dense
@@ -46,6 +48,7 @@ namespace stk {
 // hardware's dispatch through: workgroups start in order, each on the compute unit that
 // is free first.  Tiles of one kind take equally long here (the lines' average length), so
 // the compute units are kept as a few groups (free time, how many) in ascending order.
+constexpr int kSortCapacity = 4096;  // lone lines that are put in order of their lengths (more: left as they are)
 constexpr int kSimGroups = 24;    // groups alive at a time
 constexpr int kSimCapacity = 48;  // room for the queue to move along before it is shifted back
 struct DispatchSim {
@@ -201,6 +204,9 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
                                                           int compute_units, uint8_t* __restrict__ plan, int32_t* __restrict__ sdd, int max_sdd_tiles,
                                                           int sdd_rows, int sdd_cols, int most) {
   __shared__ int wave_last[16];
+  __shared__ int sort_count[256];
+  __shared__ int sort_line[kSortCapacity];
+  __shared__ uint8_t sort_key[kSortCapacity];
   __shared__ float sim_time[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
   __shared__ int sim_count[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
   const bool cols = blockIdx.x == 1;
@@ -292,6 +298,36 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
     if (most == 4) want = kind == kPairs ? 4 : kind == kTallTriples ? 3 : kind == kTallPairs ? 2 : kind == kTallSingles ? 1 : -1;
     for (int i = lo; i < hi; i++)
       if (from[i] == want) list[base++] = i;
+  }
+  // The lists of lone lines, longest first (lines of equal length keep their order): workgroups start in list order,
+  // so the long walks of an irregular pattern begin early and the short ones fill the end of the launch.  A counting
+  // sort on min(blocks, 255) in LDS; lists longer than kSortCapacity stay in ascending order.
+  {
+    const int32_t* offs = cols ? offsets_t : offsets;
+    for (int which = 0; which < 2; which++) {
+      const int kind = which ? kTallSingles : kSingles;
+      const int count = totals[kind];
+      if (count < 2 || count > kSortCapacity) continue;  // (the same for every thread)
+      int32_t* list = lists + 2 * kPlanLists + (cols ? kPlanLists * block_rows : 0) + kind * lines;
+      __syncthreads();  // the list is complete
+      if (tid < 256) sort_count[tid] = 0;
+      for (int e = tid; e < count; e += 1024) {
+        const int line = list[e], blocks = offs[line + 1] - offs[line];
+        sort_line[e] = line;
+        sort_key[e] = (uint8_t)(255 - (blocks < 255 ? blocks : 255));  // ascending key = descending length
+      }
+      __syncthreads();
+      for (int e = tid; e < count; e += 1024) atomicAdd(&sort_count[sort_key[e]], 1);
+      __syncthreads();
+      if (tid < 256 && sort_count[tid] > 0) {
+        // key `tid`: its entries go behind those of all smaller keys, in list order
+        int at = 0;
+        for (int k = 0; k < tid; k++) at += sort_count[k];
+        for (int e = 0; e < count; e++)
+          if (sort_key[e] == tid) list[at++] = sort_line[e];
+      }
+    }
+    __syncthreads();
   }
   // Tiles of stk_sdd (block rows only), row by row: groups of identical rows (sdd_rows_owned) times up to
   // sdd_cols neighbouring blocks (one for a group of three rows).

@@ -240,8 +240,11 @@ def test_fusion_plan_roles(name):
     lists = got[off:off + 4 * 5 * (2 + br + bc)].view(np.int32)
     for d, (lines, roles, talls) in enumerate([(br, got[:br], tall[:br]), (bc, got[br:br + bc], tall[br:br + bc])]):
         base = 10 + (5 * br if d else 0)
+        offs = topo.offsets_t if d else topo.offsets
         for kind, (src, want) in enumerate([(roles, 1), (roles, 0), (talls, 1), (talls, 3), (talls, 0)]):
             expect = np.nonzero(src == want)[0].tolist()
+            if want == 0:   # lone lines: longest first, equal lengths in ascending order
+                expect = _longest_first(expect, offs)
             assert int(lists[5 * d + kind]) == len(expect)
             assert lists[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
     # behind the lists, per direction: slice counts for dsd (1 .. 4) and the hint that the blocks are spread
@@ -269,13 +272,23 @@ def test_fusion_plan_roles(name):
     lists64 = both64[off:off + 4 * 5 * (2 + br + bc)].view(np.int32)
     for d, (lines, sizes) in enumerate([(br, np.array(want_rows)), (bc, np.array(want_cols))]):
         base = 10 + (5 * br if d else 0)
+        offs = topo.offsets_t if d else topo.offsets
         for kind, size in enumerate([4, None, 2, 3, 1]):
             expect = [] if size is None else np.nonzero(sizes == size)[0].tolist()
+            if size == 1:
+                expect = _longest_first(expect, offs)
             assert int(lists64[5 * d + kind]) == len(expect), (d, kind)
             assert lists64[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
     rows_only = hip_kernels.fusion_plan(_dev(topo.offsets), _dev(topo.column_indices)).cpu().numpy()
     assert rows_only[:8 + 8 * int(sdd[0])].tolist() == whole[:8 + 8 * int(sdd[0])].tolist()
     assert rows_only[sdd_bytes:sdd_bytes + br].tolist() == got[:br].tolist()
+
+
+def _longest_first(lines, offsets):
+    """Lines in order of descending min(blocks, 255), equal lengths ascending (lists of more than 4096 stay ascending)."""
+    if len(lines) > 4096:
+        return lines
+    return sorted(lines, key=lambda i: (-min(int(offsets[i + 1]) - int(offsets[i]), 255), i))
 
 
 def _groups_of_up_to_four(offsets, indices):
