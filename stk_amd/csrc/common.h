@@ -99,7 +99,10 @@ inline PlanLists plan_lists_of(const uint8_t* plan, int64_t block_rows, int64_t 
 // the dense operand) run on four-wave 128x128 tiles, two workgroups per compute unit: with so few, short tiles
 // the start and the stores of a workgroup are what counts, and a second workgroup on the unit hides them
 // (config 2, 4096^2 with 256 blocks: dsd 58 -> 53 us, dds 62 -> 52 us).
-constexpr int64_t kSmallWorkPerUnit = 40;
+#ifndef STK_SMALL_WORK_PER_UNIT
+#define STK_SMALL_WORK_PER_UNIT 40
+#endif
+constexpr int64_t kSmallWorkPerUnit = STK_SMALL_WORK_PER_UNIT;
 
 // Compute units of the current device (0 when it cannot be asked).
 inline int compute_units() {
