@@ -56,23 +56,22 @@ __global__ __launch_bounds__(512, 2) void dds_fused64_kernel(DdsArgs g, PlanList
   const int ntm = g.m / Quad::TM;
   const int quad_tiles = const_ints(plan.counts)[kPairs] * ntm, triple_tiles = const_ints(plan.counts)[kTallTriples] * ntm;
   const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntm;
-  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   int bid = blockIdx.x;
   // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, spread);
+    const int item = xcd_item(bid, pair_tiles);
     dds_tile<Pair, 64, TRANS_B, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntm], (item % ntm) * Pair::TM, smem, 2);
     return;
   }
   bid -= pair_tiles;
   if (bid < quad_tiles) {
-    const int item = xcd_item(bid, quad_tiles, spread);
+    const int item = xcd_item(bid, quad_tiles);
     dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Quad::TM, smem, 4);
     return;
   }
   bid -= quad_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles, spread);
+    const int item = xcd_item(bid, triple_tiles);
     dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntm], (item % ntm) * Quad::TM, smem, 3);
   }
 }
@@ -93,9 +92,8 @@ __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists 
     return;
   }
   const int pair_tiles = const_ints(plan.counts)[kPairs] * ntm, single_tiles = const_ints(plan.counts)[kSingles] * ntm;
-  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, spread);
+    const int item = xcd_item(bid, pair_tiles);
     dds_tile<Fused, 128, TRANS_B, true, 2>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Fused::TM, smem);
     return;
   }

@@ -58,23 +58,22 @@ __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanList
   const int ntn = g.n / Quad::TN;
   const int quad_tiles = const_ints(plan.counts)[kPairs] * ntn, triple_tiles = const_ints(plan.counts)[kTallTriples] * ntn;
   const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
-  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   int bid = blockIdx.x;
   // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, spread);
+    const int item = xcd_item(bid, pair_tiles);
     dsd_tile<Pair, 64, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Pair::TN, smem, 2);
     return;
   }
   bid -= pair_tiles;
   if (bid < quad_tiles) {
-    const int item = xcd_item(bid, quad_tiles, spread);
+    const int item = xcd_item(bid, quad_tiles);
     dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kPairs))[item / ntn], (item % ntn) * Quad::TN, smem, 4);
     return;
   }
   bid -= quad_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles, spread);
+    const int item = xcd_item(bid, triple_tiles);
     dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntn], (item % ntn) * Quad::TN, smem, 3);
   }
 }
@@ -101,15 +100,14 @@ __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists 
   const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
   const int triple_tiles = const_ints(plan.counts)[kTallTriples] * 2 * ntn;
   const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
-  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, spread);
+    const int item = xcd_item(bid, pair_tiles);
     dsd_tile<Fused, 128, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
     return;
   }
   bid -= pair_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles, spread);
+    const int item = xcd_item(bid, triple_tiles);
     dsd_tile<Triple, 128, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
     return;
   }
@@ -279,13 +277,13 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   }
   const int ordinal = item - whole;  // among the tiles of the last round: 0 .. workgroups - 1
   if (item < pair_tiles) {
-    const int i = xcd_item(item, pair_tiles, spread);
+    const int i = xcd_share(item, pair_tiles, spread);
     dsd_slice<Fused, TRANS_A, 2>(g, t, const_ints(plan.list(kTallPairs))[i / ntn], (i % ntn) * Fused::TN, slice, slices, ordinal, smem, &flag);
     return;
   }
   item -= pair_tiles;
   if (item < triple_tiles) {
-    const int i = xcd_item(item, triple_tiles, spread);
+    const int i = xcd_share(item, triple_tiles, spread);
     dsd_slice<Triple, TRANS_A, 3>(g, t, const_ints(plan.list(kTallTriples))[i / (2 * ntn)], (i % (2 * ntn)) * Triple::TN, slice, slices, ordinal, smem, &flag);
     return;
   }

@@ -721,20 +721,28 @@ __device__ __forceinline__ int xcd_chunked(int bid, int n) {
 }
 
 
-// The same for work items whose cost may drift along the list (walks of very different lengths
-// in a skewed topology): the list is cut into groups of kXcdGroup consecutive items, and each
+// The same in small portions: the list is cut into groups of GROUP consecutive items, and each
 // stretch of eight groups is spread over the eight XCDs, so that all of them move through the
-// list at the same pace while the items of a group - neighbours that share operand tiles -
-// still meet in one L2.  The tail that does not fill eight groups is taken in order.
+// list at the same pace - whatever the cost of the items does along the list (walks of very
+// different lengths in a skewed topology), and with the eight dies reading the same stretch of the
+// operands from memory at about the same time - while the items of a group, neighbours that share
+// operand tiles, still meet in one L2.  The tail that does not fill eight groups is taken in order.
 constexpr int kXcdGroup = 32;
+template <int GROUP = kXcdGroup>
 __device__ __forceinline__ int xcd_grouped(int bid, int n) {
-  constexpr int kStretch = 8 * kXcdGroup;
+  constexpr int kStretch = 8 * GROUP;
   const int base = bid / kStretch * kStretch;
   if (base + kStretch > n) return bid;
   const int r = bid - base;
-  return base + (r & 7) * kXcdGroup + (r >> 3);
+  return base + (r & 7) * GROUP + (r >> 3);
 }
-// spread (wave-uniform): small groups; otherwise eight contiguous shares.
-__device__ __forceinline__ int xcd_item(int bid, int n, bool spread) { return spread ? xcd_grouped(bid, n) : xcd_chunked(bid, n); }
+// Tiles of a plan's list of grouped lines, and the tiles of stk_sdd: groups of eight.  Measured against eight
+// contiguous shares on dMoE topologies: the same or up to 6 % faster for every product but the dsd with a sliced
+// last round, which keeps the shares (xcd_share).
+constexpr int kXcdTileGroup = 8;
+__device__ __forceinline__ int xcd_item(int bid, int n) { return xcd_grouped<kXcdTileGroup>(bid, n); }
+// spread (wave-uniform, a hint of the plan: the lines' lengths drift along the list): groups of kXcdGroup;
+// otherwise eight contiguous shares.
+__device__ __forceinline__ int xcd_share(int bid, int n, bool spread) { return spread ? xcd_grouped(bid, n) : xcd_chunked(bid, n); }
 
 }  // namespace stk

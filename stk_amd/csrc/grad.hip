@@ -22,15 +22,14 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
     const int pair_tiles = const_ints(rows.counts)[kTallPairs] * ntn;
     const int triple_tiles = const_ints(rows.counts)[kTallTriples] * 2 * ntn;
     const int single_tiles = const_ints(rows.counts)[kTallSingles] * ntn;
-    const bool spread = (const_ints(rows.hints)[kSpreadHint / 4] & 0xff) != 0;
     if (bid < pair_tiles) {
-      const int item = xcd_item(bid, pair_tiles, spread);
+      const int item = xcd_item(bid, pair_tiles);
       dsd_tile<DsdFused, 128, false, true, 2>(d, const_ints(rows.list(kTallPairs))[item / ntn], (item % ntn) * DsdFused::TN, smem);
       return;
     }
     bid -= pair_tiles;
     if (bid < triple_tiles) {
-      const int item = xcd_item(bid, triple_tiles, spread);
+      const int item = xcd_item(bid, triple_tiles);
       dsd_tile<DsdTriple, 128, false, true, 3>(d, const_ints(rows.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * DsdTriple::TN, smem);
       return;
     }
@@ -43,9 +42,8 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
     bid -= single_tiles;
   }
   const int pair_tiles = const_ints(cols.counts)[kPairs] * ntm, single_tiles = const_ints(cols.counts)[kSingles] * ntm;
-  const bool spread = (const_ints(cols.hints)[kSpreadHint / 4] & 0xff) != 0;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, spread);
+    const int item = xcd_item(bid, pair_tiles);
     dds_tile<DdsFused, 128, false, true, 2>(s, const_ints(cols.list(kPairs))[item / ntm], (item % ntm) * DdsFused::TM, smem);
     return;
   }
