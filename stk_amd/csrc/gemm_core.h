@@ -736,11 +736,21 @@ __device__ __forceinline__ int xcd_grouped(int bid, int n) {
   const int r = bid - base;
   return base + (r & 7) * GROUP + (r >> 3);
 }
-// Tiles of a plan's list of grouped lines, and the tiles of stk_sdd: groups of eight.  Measured against eight
-// contiguous shares on dMoE topologies: the same or up to 6 % faster for every product but the dsd with a sliced
-// last round, which keeps the shares (xcd_share).
-constexpr int kXcdTileGroup = 8;
-__device__ __forceinline__ int xcd_item(int bid, int n) { return xcd_grouped<kXcdTileGroup>(bid, n); }
+// Tiles of a plan's list of grouped lines (xcd_item: groups of sixteen) and the tiles of stk_sdd (xcd_tile: groups
+// of eight).  Measured against eight contiguous shares on dMoE topologies: the same or up to 6 % faster for every
+// product but the dsd with a sliced last round, which keeps the shares (xcd_share).  Equal shares of a list are
+// unequal shares of the work when the experts differ in size, and a die that lags holds the launch up.  The price
+// is operand traffic: a panel that all tiles of an expert share is fetched by every die that holds one of its
+// groups (dds on the benchmark topology: the lhs panel by four dies instead of one).  Groups of eight are another
+// 1 % faster for dds and fetch the panel eight times.
+#ifndef STK_XCD_LIST_GROUP
+#define STK_XCD_LIST_GROUP 16
+#endif
+#ifndef STK_XCD_SDD_GROUP
+#define STK_XCD_SDD_GROUP 8
+#endif
+__device__ __forceinline__ int xcd_item(int bid, int n) { return xcd_grouped<STK_XCD_LIST_GROUP>(bid, n); }
+__device__ __forceinline__ int xcd_tile(int bid, int n) { return xcd_grouped<STK_XCD_SDD_GROUP>(bid, n); }
 // spread (wave-uniform, a hint of the plan: the lines' lengths drift along the list): groups of kXcdGroup;
 // otherwise eight contiguous shares.
 __device__ __forceinline__ int xcd_share(int bid, int n, bool spread) { return spread ? xcd_grouped(bid, n) : xcd_chunked(bid, n); }

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(512, 2) void sdd_fused_kernel(SddArgs g) {
   if (g.tiles) {
     const int count = const_ints(g.tiles)[0];
     if ((int)blockIdx.x >= count) return;
-    const int item = xcd_item(blockIdx.x, count);
+    const int item = xcd_tile(blockIdx.x, count);
     const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
     const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
     const bool has1 = (shape >> 8) == 2;  // an odd row ends with a tile of one block
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(512, 2) void sdd_fused64_kernel(SddArgs g) {
   extern __shared__ __align__(16) char smem[];
   const int count = const_ints(g.tiles)[0];
   if ((int)blockIdx.x >= count) return;
-  const int item = xcd_item(blockIdx.x, count);
+  const int item = xcd_tile(blockIdx.x, count);
   const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
   const int rows = shape & 0xff, cols = shape >> 8;
   const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
