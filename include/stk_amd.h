@@ -86,9 +86,9 @@ int stk_abi_version(void);
  * the next two lines), then as int32 ten counts and ten lists of the lines that
  * own a tile (per direction: role 1, role 0, and with groups of three 1, 3, 0), from which
  * stk_dsd and stk_dds take their work, and 2 x 32 bytes of hints for their launches.  The
- * lists of grouped lines ascend; the two lists of lone lines (role 0) are in order of
- * descending length (lengths above 255 blocks count as 255; ties and lists of more than
- * 4096 lines ascend), so that a launch starts its longest walks first.
+ * lists are in order of descending length of their lines (lengths above 255 blocks count
+ * as 255; ties, and lists of more than 4096 lines, ascend), so that a launch starts its
+ * longest walks first wherever they lie in the matrix.
  * A plan built with blocking 64 groups the lines by fours instead of pairs (lists: first lines of groups of four,
  * none, of pairs, of groups of three, lone lines; lines too long for a compute unit's share are cut into pairs); a
  * plan must be passed only to products with the blocking it was built with.

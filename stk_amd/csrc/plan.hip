@@ -299,17 +299,18 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
     for (int i = lo; i < hi; i++)
       if (from[i] == want) list[base++] = i;
   }
-  // The lists of lone lines, longest first (lines of equal length keep their order): workgroups start in list order,
-  // so the long walks of an irregular pattern begin early and the short ones fill the end of the launch.  A counting
-  // sort on min(blocks, 255) in LDS; lists longer than kSortCapacity stay in ascending order.
+  // Every list longest first (lines of equal length keep their order, so the lines of an expert stay neighbours):
+  // workgroups start in list order, so the long walks begin early and the short ones fill the end of the launch,
+  // wherever the long lines lie in the matrix.  A counting sort on min(blocks, 255) in LDS; a list that is in this
+  // order already (all lines equally long: the block rows of a dMoE topology) is left alone, lists longer than
+  // kSortCapacity stay in ascending order.
   {
     const int32_t* offs = cols ? offsets_t : offsets;
-    for (int which = 0; which < 2; which++) {
-      const int kind = which ? kTallSingles : kSingles;
+    for (int kind = 0; kind < kPlanLists; kind++) {
       const int count = totals[kind];
       if (count < 2 || count > kSortCapacity) continue;  // (the same for every thread)
       int32_t* list = lists + 2 * kPlanLists + (cols ? kPlanLists * block_rows : 0) + kind * lines;
-      __syncthreads();  // the list is complete
+      __syncthreads();  // the list is complete, the last sort is over
       if (tid < 256) sort_count[tid] = 0;
       for (int e = tid; e < count; e += 1024) {
         const int line = list[e], blocks = offs[line + 1] - offs[line];
@@ -317,14 +318,17 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
         sort_key[e] = (uint8_t)(255 - (blocks < 255 ? blocks : 255));  // ascending key = descending length
       }
       __syncthreads();
+      int unordered = 0;
+      for (int e = tid; e + 1 < count; e += 1024) unordered |= sort_key[e] > sort_key[e + 1];
+      if (__syncthreads_or(unordered) == 0) continue;
       for (int e = tid; e < count; e += 1024) atomicAdd(&sort_count[sort_key[e]], 1);
       __syncthreads();
       if (tid < 256 && sort_count[tid] > 0) {
         // key `tid`: its entries go behind those of all smaller keys, in list order
-        int at = 0;
+        int at = 0, left = sort_count[tid];
         for (int k = 0; k < tid; k++) at += sort_count[k];
-        for (int e = 0; e < count; e++)
-          if (sort_key[e] == tid) list[at++] = sort_line[e];
+        for (int e = 0; left > 0; e++)
+          if (sort_key[e] == tid) list[at++] = sort_line[e], left--;
       }
     }
     __syncthreads();

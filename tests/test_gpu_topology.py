@@ -235,7 +235,7 @@ def test_fusion_plan_roles(name):
     tall = got[2 * (br + bc):]
     assert tall[:br].tolist() == _greedy_roles_with_threes(topo.offsets, topo.column_indices)
     assert tall[br:br + bc].tolist() == _greedy_roles_with_threes(topo.offsets_t, topo.column_indices_t)
-    # behind the roles: ten counts, then five ascending lists per direction (role 1, role 0, tall 1, tall 3, tall 0)
+    # behind the roles: ten counts, then five lists per direction (role 1, role 0, tall 1, tall 3, tall 0), longest lines first
     off = (3 * (br + bc) + 3) // 4 * 4
     lists = got[off:off + 4 * 5 * (2 + br + bc)].view(np.int32)
     for d, (lines, roles, talls) in enumerate([(br, got[:br], tall[:br]), (bc, got[br:br + bc], tall[br:br + bc])]):
@@ -243,8 +243,7 @@ def test_fusion_plan_roles(name):
         offs = topo.offsets_t if d else topo.offsets
         for kind, (src, want) in enumerate([(roles, 1), (roles, 0), (talls, 1), (talls, 3), (talls, 0)]):
             expect = np.nonzero(src == want)[0].tolist()
-            if want == 0:   # lone lines: longest first, equal lengths in ascending order
-                expect = _longest_first(expect, offs)
+            expect = _longest_first(expect, offs)   # every list: longest first, equal lengths in ascending order
             assert int(lists[5 * d + kind]) == len(expect)
             assert lists[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
     # behind the lists, per direction: slice counts for dsd (1 .. 4) and the hint that the blocks are spread
@@ -275,8 +274,7 @@ def test_fusion_plan_roles(name):
         offs = topo.offsets_t if d else topo.offsets
         for kind, size in enumerate([4, None, 2, 3, 1]):
             expect = [] if size is None else np.nonzero(sizes == size)[0].tolist()
-            if size == 1:
-                expect = _longest_first(expect, offs)
+            expect = _longest_first(expect, offs)
             assert int(lists64[5 * d + kind]) == len(expect), (d, kind)
             assert lists64[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
     rows_only = hip_kernels.fusion_plan(_dev(topo.offsets), _dev(topo.column_indices)).cpu().numpy()
