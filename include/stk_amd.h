@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 9
+#define STK_AMD_ABI_VERSION 10
 
 /* status codes */
 #define STK_OK 0
@@ -269,15 +269,37 @@ int stk_to_dense(const void* data, const void* row_indices, const void* column_i
  *          blocks and data[nnz, b, b] gathered from x; nnz is the value read
  *          back after count.
  * x is [rows, cols] row-major with leading dimension x_stride; elem_bytes 2 or 4.
+ * stk_to_sparse_count_nnz also stores nnz at nnz_out (NULL: not stored) as the last thing
+ * the launch does, with a system-scope release store; nnz_out may be device memory or pinned
+ * host memory that the device can write.  A caller that set the word to a value nnz cannot
+ * take (-1) before the call may poll it from the host instead of waiting for the stream;
+ * offsets and mask are complete in device memory when the value appears.
  */
 int stk_to_sparse_count(const void* x, int64_t rows, int64_t cols, int64_t x_stride,
                         int blocking, int elem_bytes,
                         uint8_t* mask, int32_t* offsets, stk_stream_t stream);
+int stk_to_sparse_count_nnz(const void* x, int64_t rows, int64_t cols, int64_t x_stride,
+                            int blocking, int elem_bytes,
+                            uint8_t* mask, int32_t* offsets, int32_t* nnz_out, stk_stream_t stream);
 int stk_to_sparse_fill(const void* x, int64_t rows, int64_t cols, int64_t x_stride,
                        int blocking, int elem_bytes,
                        const uint8_t* mask, const int32_t* offsets, int64_t nnz,
                        void* data, void* row_indices, void* column_indices,
                        int index_dtype, stk_stream_t stream);
+/*
+ * The two halves of stk_to_sparse_fill on their own.  The coordinates depend on mask and
+ * offsets only, not on nnz read back by the host: a caller that has room for Rb*Cb indices
+ * can launch them behind the count, before it waits for nnz, and has only the gather of the
+ * values left to launch afterwards (row_indices / column_indices: the first nnz entries are
+ * written).
+ */
+int stk_to_sparse_coordinates(int64_t rows, int64_t cols, int blocking,
+                              const uint8_t* mask, const int32_t* offsets,
+                              void* row_indices, void* column_indices, int index_dtype, stk_stream_t stream);
+int stk_to_sparse_gather(const void* x, int64_t rows, int64_t cols, int64_t x_stride,
+                         int blocking, int elem_bytes,
+                         const void* row_indices, const void* column_indices, int64_t nnz,
+                         int index_dtype, void* data, stk_stream_t stream);
 
 /*
  * Topology of a dropless mixture-of-experts layer, built in one launch from the

@@ -11,7 +11,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
 STK_F16, STK_BF16 = 0, 1
 STK_I16, STK_I32 = 0, 1
@@ -39,7 +39,10 @@ SIGNATURES = {
     "stk_transpose_meta": (_int, [_p, _p, _i64, _i64, _int, _p, _p, _p, _p, _sz, _p]),
     "stk_to_dense": (_int, [_p, _p, _p, _i64, _int, _i64, _i64, _int, _int, _p, _p]),
     "stk_to_sparse_count": (_int, [_p, _i64, _i64, _i64, _int, _int, _p, _p, _p]),
+    "stk_to_sparse_count_nnz": (_int, [_p, _i64, _i64, _i64, _int, _int, _p, _p, _p, _p]),
     "stk_to_sparse_fill": (_int, [_p, _i64, _i64, _i64, _int, _int, _p, _p, _i64, _p, _p, _p, _int, _p]),
+    "stk_to_sparse_coordinates": (_int, [_i64, _i64, _int, _p, _p, _p, _p, _int, _p]),
+    "stk_to_sparse_gather": (_int, [_p, _i64, _i64, _i64, _int, _int, _p, _p, _i64, _int, _p, _p]),
     "stk_dmoe_topology": (_int, [_p, _i64, _int, _i64, _i64, _int, _p, _p, _p, _p, _p, _p, _p]),
     "stk_route_workspace_bytes": (_sz, [_i64, _i64]),
     "stk_route": (_int, [_p, _i64, _i64, _int, _i64, _p, _p, _p, _p, _p, _p, _p, _sz, _p]),

@@ -11,6 +11,8 @@ Everything here needs tensors on a ROCm device and launches on torch's current
 stream without synchronising (to_sparse reads one int back, as the reference's
 torch.nonzero does).  Nothing falls back to another implementation.
 """
+import threading
+
 import torch
 
 from stk_amd.backend import _lib
@@ -410,6 +412,10 @@ def to_dense(data, row_indices, column_indices, rows, cols):
     return out
 
 
+NNZ_POLL_LIMIT = 200000   # polls of the pinned nnz word (some 20 ms) before to_sparse waits for the stream instead
+_nnz_buffers = threading.local()   # per host thread: device index -> pinned int32[1] that stk_to_sparse_count_nnz writes nnz into
+
+
 def to_sparse(x, blocking, index_dtype=torch.int16):
     """(data, row_indices, column_indices, offsets) of the nonzero blocks of x."""
     _need_gpu(x)
@@ -421,19 +427,41 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
     x = x.detach()
     br, bc = rows // blocking, cols // blocking
     dev = x.device
-    mask = torch.empty(max(br * bc, 1), dtype=torch.uint8, device=dev)
-    offsets = torch.empty(br + 1, dtype=torch.int32, device=dev)
+    # one allocation for offsets (int32) and the block mask (bytes) behind it
+    scratch = torch.empty(4 * (br + 1) + max(br * bc, 1), dtype=torch.uint8, device=dev)
+    offsets, mask = scratch[:4 * (br + 1)].view(torch.int32), scratch[4 * (br + 1):]
     lib = _lib.load()
     with _on_device(dev):
-        _lib.check(lib.stk_to_sparse_count(
-            x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), mask.data_ptr(), offsets.data_ptr(), _stream()))
-        nnz = int(offsets[-1].item())
+        # nnz arrives in pinned host memory, written by the counting kernel: one wait, no copy to launch
+        buffers = _nnz_buffers.__dict__.setdefault("of_device", {})
+        nnz_host = buffers.get(dev.index)
+        if nnz_host is None:
+            nnz_host = buffers[dev.index] = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        word = nnz_host.numpy()
+        word[0] = -1
+        _lib.check(lib.stk_to_sparse_count_nnz(
+            x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), mask.data_ptr(), offsets.data_ptr(), nnz_host.data_ptr(),
+            _stream()))
+        # the coordinates need no nnz: launched behind the count, into room for every block (the first nnz entries
+        # are written; the index tensors returned are views of that room)
+        room = torch.empty(2 * max(br * bc, 1), dtype=index_dtype, device=dev)
+        _lib.check(lib.stk_to_sparse_coordinates(rows, cols, blocking, mask.data_ptr(), offsets.data_ptr(), room.data_ptr(),
+                                                 room.data_ptr() + br * bc * room.element_size(), _INDEX_DTYPES[index_dtype], _stream()))
+        # the counting kernel's last store is nnz: poll the pinned word instead of sleeping in a stream wait (whose
+        # wake-up costs more than the kernels of a small matrix); after a while fall back to the wait, which also
+        # reports a launch that failed
+        spins = 0
+        while word[0] < 0 and spins < NNZ_POLL_LIMIT:
+            spins += 1
+        if word[0] < 0:
+            torch.cuda.current_stream(dev).synchronize()
+            assert word[0] >= 0, "stk_to_sparse_count_nnz did not deliver nnz"
+        nnz = int(word[0])
+        row_indices, column_indices = room[:nnz], room[br * bc:br * bc + nnz]
         data = torch.empty((nnz, blocking, blocking), dtype=x.dtype, device=dev)
-        row_indices = torch.empty(nnz, dtype=index_dtype, device=dev)
-        column_indices = torch.empty(nnz, dtype=index_dtype, device=dev)
-        _lib.check(lib.stk_to_sparse_fill(
-            x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), mask.data_ptr(), offsets.data_ptr(), nnz,
-            data.data_ptr(), row_indices.data_ptr(), column_indices.data_ptr(), _INDEX_DTYPES[index_dtype], _stream()))
+        _lib.check(lib.stk_to_sparse_gather(
+            x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), row_indices.data_ptr(), column_indices.data_ptr(), nnz,
+            _INDEX_DTYPES[index_dtype], data.data_ptr(), _stream()))
     return data, row_indices, column_indices, offsets
 
 

@@ -346,7 +346,8 @@ __global__ __launch_bounds__(256) void block_mask_kernel(const E* __restrict__ x
 }
 
 // The same with 16 bytes per lane, for blocks whose rows are a power-of-two number (at most 64) of aligned
-// 16-byte pieces: a wavefront covers 64 >> log2_pieces block rows per load and keeps four loads in flight.
+// 16-byte pieces: a wavefront covers 64 >> log2_pieces block rows per load, keeps four and then eight loads in flight,
+// and reads no further when the first four loads hold a nonzero element.
 template <int ELEM_BYTES>
 __global__ __launch_bounds__(256) void block_mask_vec_kernel(const char* __restrict__ x, int64_t ld_bytes, int b, int log2_pieces,
                                                              int block_cols, int64_t blocks, uint8_t* __restrict__ mask) {
@@ -361,17 +362,22 @@ __global__ __launch_bounds__(256) void block_mask_vec_kernel(const char* __restr
     const int64_t r = blk / block_cols, c = blk - r * block_cols;
     const char* base = x + r * b * ld_bytes + c * (int64_t)b * ELEM_BYTES + lane_offset;
     uint32_t any = 0;
-    for (int i0 = 0; i0 < b; i0 += 4 * rows_per_load) {
-      uint4 v[4];
+    // The first four loads decide for almost every nonzero block; a block that is zero so far is read to its end,
+    // eight loads in flight, with nothing to wait for between the steps.
+    auto read = [&](int i0, int loads) {
+      uint4 v[8];
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
+      for (int u = 0; u < 8; u++) {
         const int i = i0 + u * rows_per_load + row0;
         v[u] = make_uint4(0u, 0u, 0u, 0u);
-        if (i < b) v[u] = *reinterpret_cast<const uint4*>(base + (int64_t)(i0 + u * rows_per_load) * ld_bytes);
+        if (u < loads && i < b) v[u] = *reinterpret_cast<const uint4*>(base + (int64_t)(i0 + u * rows_per_load) * ld_bytes);
       }
 #pragma unroll
-      for (int u = 0; u < 4; u++) any |= (v[u].x | v[u].y | v[u].z | v[u].w) & kAbs;
-    }
+      for (int u = 0; u < 8; u++) any |= (v[u].x | v[u].y | v[u].z | v[u].w) & kAbs;
+    };
+    read(0, 4);
+    if (__ballot(any != 0) == 0)
+      for (int i0 = 4 * rows_per_load; i0 < b; i0 += 8 * rows_per_load) read(i0, 8);
     const uint64_t bal = __ballot(any != 0);
     if (lane == 0) mask[blk] = bal != 0;
   }
@@ -380,7 +386,7 @@ __global__ __launch_bounds__(256) void block_mask_vec_kernel(const char* __restr
 // offsets[0] = 0, offsets[r + 1] = number of nonzero blocks in rows 0..r.  One workgroup; a wavefront counts a
 // block row at a time (coalesced reads of the mask), sixteen rows per round, then a scan over the rounds' counts.
 __global__ __launch_bounds__(1024) void row_offsets_kernel(const uint8_t* __restrict__ mask, int block_rows, int block_cols,
-                                                           int32_t* __restrict__ offsets) {
+                                                           int32_t* __restrict__ offsets, int32_t* __restrict__ total_out) {
   __shared__ int part[16];
   __shared__ int counts[1024];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -402,6 +408,10 @@ __global__ __launch_bounds__(1024) void row_offsets_kernel(const uint8_t* __rest
     if (r < block_rows) offsets[r + 1] = carry + ex + cnt;
     carry += total;
     __syncthreads();
+  }
+  if (total_out && threadIdx.x == 0) {
+    // (may be pinned host memory that the host polls: a system-scope store, made visible at once)
+    __hip_atomic_store(total_out, carry, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -551,6 +561,11 @@ extern "C" int stk_to_dense(const void* data, const void* row_indices, const voi
 
 extern "C" int stk_to_sparse_count(const void* x, int64_t rows, int64_t cols, int64_t x_stride, int blocking, int elem_bytes,
                                    uint8_t* mask, int32_t* offsets, stk_stream_t stream) {
+  return stk_to_sparse_count_nnz(x, rows, cols, x_stride, blocking, elem_bytes, mask, offsets, nullptr, stream);
+}
+
+extern "C" int stk_to_sparse_count_nnz(const void* x, int64_t rows, int64_t cols, int64_t x_stride, int blocking, int elem_bytes,
+                                       uint8_t* mask, int32_t* offsets, int32_t* nnz_out, stk_stream_t stream) {
   if (elem_bytes != 2 && elem_bytes != 4) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_count: element size %d", elem_bytes);
   if (blocking <= 0 || rows < 0 || cols < 0 || rows % blocking || cols % blocking)
     return fail(STK_ERR_DIMS, "stk_to_sparse_count: [%lld, %lld] is not divisible by blocking %d", (long long)rows, (long long)cols, blocking);
@@ -579,19 +594,18 @@ extern "C" int stk_to_sparse_count(const void* x, int64_t rows, int64_t cols, in
     else
       hipLaunchKernelGGL((block_mask_kernel<uint32_t>), dim3(grid), dim3(256), 0, s, static_cast<const uint32_t*>(x), x_stride, blocking, (int)bc, blocks, mask);
   }
-  hipLaunchKernelGGL(row_offsets_kernel, dim3(1), dim3(1024), 0, s, mask, (int)br, (int)bc, offsets);
+  hipLaunchKernelGGL(row_offsets_kernel, dim3(1), dim3(1024), 0, s, mask, (int)br, (int)bc, offsets, nnz_out);
   return check_launch("stk_to_sparse_count");
 }
 
-extern "C" int stk_to_sparse_fill(const void* x, int64_t rows, int64_t cols, int64_t x_stride, int blocking, int elem_bytes,
-                                  const uint8_t* mask, const int32_t* offsets, int64_t nnz, void* data, void* row_indices,
-                                  void* column_indices, int index_dtype, stk_stream_t stream) {
-  if (elem_bytes != 2 && elem_bytes != 4) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_fill: element size %d", elem_bytes);
-  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_fill: index dtype %d", index_dtype);
+extern "C" int stk_to_sparse_coordinates(int64_t rows, int64_t cols, int blocking, const uint8_t* mask, const int32_t* offsets,
+                                         void* row_indices, void* column_indices, int index_dtype, stk_stream_t stream) {
+  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_coordinates: index dtype %d", index_dtype);
   if (blocking <= 0 || rows < 0 || cols < 0 || rows % blocking || cols % blocking)
-    return fail(STK_ERR_DIMS, "stk_to_sparse_fill: [%lld, %lld] is not divisible by blocking %d", (long long)rows, (long long)cols, blocking);
+    return fail(STK_ERR_DIMS, "stk_to_sparse_coordinates: [%lld, %lld] is not divisible by blocking %d", (long long)rows, (long long)cols, blocking);
   const int64_t br = rows / blocking, bc = cols / blocking;
-  if (br == 0 || bc == 0 || nnz <= 0) return STK_OK;
+  if (br == 0 || bc == 0) return STK_OK;
+  if (br > INT32_MAX || bc > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_coordinates: size exceeds 32-bit range");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = (int)((br + 3) / 4 < 65536 ? (br + 3) / 4 : 65536);
   if (index_dtype == STK_I32)
@@ -600,10 +614,29 @@ extern "C" int stk_to_sparse_fill(const void* x, int64_t rows, int64_t cols, int
   else
     hipLaunchKernelGGL((block_coordinates_kernel<int16_t>), dim3(grid), dim3(256), 0, s, mask, offsets, (int)br, (int)bc,
                        static_cast<int16_t*>(row_indices), static_cast<int16_t*>(column_indices));
-  int rc = check_launch("stk_to_sparse_fill");
-  if (rc) return rc;
+  return check_launch("stk_to_sparse_coordinates");
+}
+
+extern "C" int stk_to_sparse_gather(const void* x, int64_t rows, int64_t cols, int64_t x_stride, int blocking, int elem_bytes,
+                                    const void* row_indices, const void* column_indices, int64_t nnz, int index_dtype, void* data,
+                                    stk_stream_t stream) {
+  if (elem_bytes != 2 && elem_bytes != 4) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_gather: element size %d", elem_bytes);
+  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_gather: index dtype %d", index_dtype);
+  if (blocking <= 0 || rows < 0 || cols < 0 || rows % blocking || cols % blocking)
+    return fail(STK_ERR_DIMS, "stk_to_sparse_gather: [%lld, %lld] is not divisible by blocking %d", (long long)rows, (long long)cols, blocking);
+  if (rows == 0 || cols == 0 || nnz <= 0) return STK_OK;
   return block_copy<false>(data, const_cast<void*>(x), row_indices, column_indices, nnz, blocking, x_stride, elem_bytes,
-                           index_dtype == STK_I32, s);
+                           index_dtype == STK_I32, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int stk_to_sparse_fill(const void* x, int64_t rows, int64_t cols, int64_t x_stride, int blocking, int elem_bytes,
+                                  const uint8_t* mask, const int32_t* offsets, int64_t nnz, void* data, void* row_indices,
+                                  void* column_indices, int index_dtype, stk_stream_t stream) {
+  if (elem_bytes != 2 && elem_bytes != 4) return fail(STK_ERR_UNSUPPORTED, "stk_to_sparse_fill: element size %d", elem_bytes);
+  if (nnz <= 0) return STK_OK;
+  const int rc = stk_to_sparse_coordinates(rows, cols, blocking, mask, offsets, row_indices, column_indices, index_dtype, stream);
+  if (rc != STK_OK) return rc;
+  return stk_to_sparse_gather(x, rows, cols, x_stride, blocking, elem_bytes, row_indices, column_indices, nnz, index_dtype, data, stream);
 }
 
 extern "C" int stk_dmoe_topology(const int32_t* padded_bins, int64_t num_experts, int blocking, int64_t block_rows,
