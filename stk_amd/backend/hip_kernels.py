@@ -444,9 +444,10 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
             _stream()))
         # the coordinates need no nnz: launched behind the count, into room for every block (the first nnz entries
         # are written; the index tensors returned are views of that room)
-        room = torch.empty(2 * max(br * bc, 1), dtype=index_dtype, device=dev)
+        half = (br * bc + 127) // 128 * 128   # (both index arrays start at a multiple of 256 bytes, like allocations of their own)
+        room = torch.empty(2 * max(half, 128), dtype=index_dtype, device=dev)
         _lib.check(lib.stk_to_sparse_coordinates(rows, cols, blocking, mask.data_ptr(), offsets.data_ptr(), room.data_ptr(),
-                                                 room.data_ptr() + br * bc * room.element_size(), _INDEX_DTYPES[index_dtype], _stream()))
+                                                 room.data_ptr() + half * room.element_size(), _INDEX_DTYPES[index_dtype], _stream()))
         # the counting kernel's last store is nnz: poll the pinned word instead of sleeping in a stream wait (whose
         # wake-up costs more than the kernels of a small matrix); after a while fall back to the wait, which also
         # reports a launch that failed
@@ -457,7 +458,7 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
             torch.cuda.current_stream(dev).synchronize()
             assert word[0] >= 0, "stk_to_sparse_count_nnz did not deliver nnz"
         nnz = int(word[0])
-        row_indices, column_indices = room[:nnz], room[br * bc:br * bc + nnz]
+        row_indices, column_indices = room[:nnz], room[half:half + nnz]
         data = torch.empty((nnz, blocking, blocking), dtype=x.dtype, device=dev)
         _lib.check(lib.stk_to_sparse_gather(
             x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), row_indices.data_ptr(), column_indices.data_ptr(), nnz,
