@@ -468,9 +468,11 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
     constexpr int NKS = Cfg::KT / 16;
     constexpr int kMfmas = Cfg::IM * Cfg::JN;
     constexpr int kPiecesPerMfma = (kLoadsPerTile + kMfmas - 1) / kMfmas;
-    static_assert(NKS % 2 == 0 && S <= 4, "fragment buffers alternate per k-step; the waits below cover three or four stages");
+    static_assert(NKS % 2 == 0 && S <= 5, "fragment buffers alternate per k-step; the waits below cover three to five stages");
     if (ntiles > 0) {
-      if (S >= 4 && ntiles >= 3) wait_vmcnt<2 * kLoadsPerTile>();
+      // K-tile 0 must have landed; the younger ones of the first S - 1 may stay in flight
+      if (S >= 5 && ntiles >= 4) wait_vmcnt<3 * kLoadsPerTile>();
+      else if (S >= 4 && ntiles >= 3) wait_vmcnt<2 * kLoadsPerTile>();
       else if (ntiles >= 2) wait_vmcnt<1 * kLoadsPerTile>();
       else wait_vmcnt<0>();
       __syncthreads();
@@ -501,7 +503,9 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
         if constexpr (REFILL) {
           wait_vmcnt<(S - 3) * kLoadsPerTile>();
         } else {
-          if (S >= 4 && t + 2 < ntiles) wait_vmcnt<(S - 3) * kLoadsPerTile>();
+          // no refill any more: K-tiles t + 2 .. ntiles - 1 (at most S - 3 of them) are still in flight
+          if (S >= 5 && t + 3 < ntiles) wait_vmcnt<2 * kLoadsPerTile>();
+          else if (S >= 4 && t + 2 < ntiles) wait_vmcnt<1 * kLoadsPerTile>();
           else wait_vmcnt<0>();
         }
         __syncthreads();
