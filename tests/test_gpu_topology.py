@@ -201,7 +201,7 @@ def _greedy_roles_with_threes(offsets, indices):
     return role
 
 
-@pytest.mark.parametrize("name", ["dmoe", "skewed", "random", "dense", "empty", "runs"])
+@pytest.mark.parametrize("name", ["dmoe", "skewed", "random", "dense", "empty", "runs", "many", "tall"])
 def test_fusion_plan_roles(name):
     if name == "dmoe":
         topo = O.dmoe_topology([300, 0, 129, 1, 640, 128, 77, 256, 512], 512, 128)
@@ -215,6 +215,10 @@ def test_fusion_plan_roles(name):
             mask = np.ones((9, 5), bool)
         elif name == "empty":
             mask = np.zeros((6, 4), bool)
+        elif name == "many":    # more lone rows than the plan sorts (they stay ascending); columns of about 100 blocks
+            mask = rng.rand(5000, 300) < 0.02
+        elif name == "tall":    # columns of more than 255 blocks: equal keys, ascending among themselves
+            mask = rng.rand(600, 7) < 0.7
         else:   # runs of 1..5 identical rows, some empty rows in between
             rows = []
             for n in [1, 2, 3, 4, 5, 2, 1, 3, 9, 6]:
