@@ -17,6 +17,10 @@
 #define STK_DSD_KT 32
 #define STK_DSD_STAGES 4
 #endif
+#ifndef STK_DSD_BK_KT
+#define STK_DSD_BK_KT 64   // K-major dense operand
+#define STK_DSD_BK_STAGES 2
+#endif
 #ifndef STK_DSD_T_KT
 #define STK_DSD_T_KT 32
 #define STK_DSD_T_STAGES 4

@@ -311,7 +311,7 @@ template <bool BF16, int BLK, bool TRANS_A, bool BK, bool STREAM>
 static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* tail, hipStream_t stream) {
   // K-major dense operand (a .t() view): a 32-deep K-tile would use half of every 128-byte line it touches, so
   // 64-deep K-tiles (two stages fit) beat the deeper ring of 32-deep ones
-  constexpr int KT = BK ? 64 : (TRANS_A ? STK_DSD_T_KT : STK_DSD_KT), S = BK ? 2 : (TRANS_A ? STK_DSD_T_STAGES : STK_DSD_STAGES);
+  constexpr int KT = BK ? STK_DSD_BK_KT : (TRANS_A ? STK_DSD_T_KT : STK_DSD_KT), S = BK ? STK_DSD_BK_STAGES : (TRANS_A ? STK_DSD_T_STAGES : STK_DSD_STAGES);
   if constexpr (BLK == 128) {
     // eight wavefronts: 4x2 of 64x128 over two block rows, or 2x4 of 64x64 over one
     using Fused = TileCfg<4, 2, 2, 4, 1, 2, 2, !TRANS_A, BK, BF16, KT, S, false, STREAM>;
