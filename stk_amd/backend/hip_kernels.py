@@ -21,8 +21,17 @@ _VALUE_DTYPES = {torch.float16: _lib.STK_F16, torch.bfloat16: _lib.STK_BF16}
 _INDEX_DTYPES = {torch.int16: _lib.STK_I16, torch.int32: _lib.STK_I32}
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def _stream(device=None):
+    """Handle of torch's current stream on `device` (default: the current device).  Read through torch's C entry
+    points where they exist: torch.cuda.current_stream() builds a Stream object, which costs several microseconds
+    on a path that every launch takes."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device() if device is None or device.index is None else device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 class _on_device:
@@ -30,7 +39,8 @@ class _on_device:
     already is (the usual case, and this sits on the launch path of every product)."""
 
     def __init__(self, device):
-        self._guard = None if device.index is None or device.index == torch.cuda.current_device() else torch.cuda.device(device)
+        current = _raw_device() if _raw_device is not None else torch.cuda.current_device()
+        self._guard = None if device.index is None or device.index == current else torch.cuda.device(device)
 
     def __enter__(self):
         if self._guard is not None:
@@ -142,9 +152,9 @@ def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, 
     tensors = (offsets, column_indices) + ((offsets_t, column_indices_t) if want_cols else ())
     cached = _plan_cache_get(tensors, blocking)
     if cached is not None:
-        stream = torch.cuda.current_stream(offsets.device)
-        if cached[3] != stream.cuda_stream:
-            stream.wait_event(cached[4])  # built on another stream: what this one launches next comes after the build
+        if cached[3] != _stream(offsets.device):
+            # built on another stream: what this one launches next comes after the build
+            torch.cuda.current_stream(offsets.device).wait_event(cached[4])
         return cached[1]
     block_rows = offsets.numel() - 1
     block_cols = offsets_t.numel() - 1 if want_cols else 0
@@ -244,16 +254,17 @@ def _dsd_workspace(device, m, n, blocking):
     lib = _lib.load()
     if lib.stk_dsd_workspace_bytes(m, n, blocking) <= 0:
         return None
-    stream = torch.cuda.current_stream(device)
-    key = (device.index, stream.cuda_stream in CONCURRENT_STREAMS)
+    handle = _stream(device)
+    key = (device.index, handle in CONCURRENT_STREAMS)
     entry = _dsd_workspaces.get(key)
     counters = lib.stk_dsd_workspace_counter_bytes()
     nbytes = counters + DSD_WORKSPACE_SLOTS * lib.stk_dsd_workspace_slot_bytes()
     if entry is None or entry[0].numel() != nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
         ws[:counters].zero_()   # the slots behind the counters need no initial value
-        entry = _dsd_workspaces[key] = [ws, stream]
-    elif entry[1].cuda_stream != stream.cuda_stream:
+        entry = _dsd_workspaces[key] = [ws, torch.cuda.current_stream(device)]
+    elif entry[1].cuda_stream != handle:
+        stream = torch.cuda.current_stream(device)
         stream.wait_stream(entry[1])   # launches that share a workspace must not overlap
         entry[1] = stream
     return entry[0]
