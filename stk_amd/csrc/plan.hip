@@ -38,6 +38,7 @@
 //   list 2 (tall 1's place)  of pairs                           list 4 (tall 0's place)  lone lines
 // with list 1 empty.
 #include "common.h"
+#include "wave_scan.h"
 
 namespace stk {
 
@@ -207,6 +208,7 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
   __shared__ int sort_count[256];
   __shared__ int sort_line[kSortCapacity];
   __shared__ uint8_t sort_key[kSortCapacity];
+  __shared__ uint16_t sort_wave[16 * 256];  // per wavefront and key: a count, then the place of the first such entry
   __shared__ float sim_time[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
   __shared__ int sim_count[kTailSliceColumns * kMaxTailSlices][kSimCapacity];
   const bool cols = blockIdx.x == 1;
@@ -323,12 +325,43 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
       if (__syncthreads_or(unordered) == 0) continue;
       for (int e = tid; e < count; e += 1024) atomicAdd(&sort_count[sort_key[e]], 1);
       __syncthreads();
-      if (tid < 256 && sort_count[tid] > 0) {
-        // key `tid`: its entries go behind those of all smaller keys, in list order
-        int at = 0, left = sort_count[tid];
-        for (int k = 0; k < tid; k++) at += sort_count[k];
-        for (int e = 0; left > 0; e++)
-          if (sort_key[e] == tid) list[at++] = sort_line[e], left--;
+      // sort_count[k]: where the entries with key k begin (an exclusive scan over the keys)
+      {
+        int total;
+        const int begin = block_exclusive_scan(tid < 256 ? sort_count[tid] : 0, wave_last, &total);
+        if (tid < 256) sort_count[tid] = begin;
+      }
+      // 1024 entries at a time, in list order: an entry goes behind the entries with its key that came before it -
+      // those of earlier rounds (sort_count runs on), of earlier wavefronts of this round (sort_wave) and of
+      // earlier lanes of its wavefront (counted with ballots, one distinct key of the wavefront at a time)
+      for (int e0 = 0; e0 < count; e0 += 1024) {
+        for (int i = tid; i < 16 * 256; i += 1024) sort_wave[i] = 0;
+        __syncthreads();
+        const int e = e0 + tid;
+        const bool valid = e < count;
+        const int key = valid ? sort_key[e] : -1;
+        int rank = 0;
+        uint64_t todo = __ballot(valid);
+        while (todo) {
+          const int k = __builtin_amdgcn_readlane(key, __ffsll((unsigned long long)todo) - 1);
+          const uint64_t same = __ballot(key == k);
+          if (key == k) rank = __popcll(same & ((1ull << lane) - 1));
+          if (lane == 0) sort_wave[wave * 256 + k] = (uint16_t)__popcll(same);
+          todo &= ~same;
+        }
+        __syncthreads();
+        if (tid < 256) {
+          int at = sort_count[tid];
+          for (int w = 0; w < 16; w++) {
+            const int n = sort_wave[w * 256 + tid];
+            sort_wave[w * 256 + tid] = (uint16_t)at;
+            at += n;
+          }
+          sort_count[tid] = at;
+        }
+        __syncthreads();
+        if (valid) list[sort_wave[wave * 256 + key] + rank] = sort_line[e];
+        __syncthreads();
       }
     }
     __syncthreads();
