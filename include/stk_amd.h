@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 10
+#define STK_AMD_ABI_VERSION 11
 
 /* status codes */
 #define STK_OK 0
@@ -61,6 +61,12 @@ extern "C" {
 #define STK_ACT_GELU_TANH 2 /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) */
 #define STK_ACT_GELU 3      /* 0.5 x (1 + erf(x / sqrt 2)) */
 #define STK_ACT_SILU 4      /* x / (1 + exp(-x)) */
+/* the derivatives of the four: with the incoming gradient as the multiplier, stk_sdd_fused then yields the gradient with
+ * respect to the sums of a stk_sdd_fused that applied the function, in the one pass that recomputes the sums */
+#define STK_ACT_RELU_GRAD 5
+#define STK_ACT_GELU_TANH_GRAD 6
+#define STK_ACT_GELU_GRAD 7
+#define STK_ACT_SILU_GRAD 8
 
 typedef void* stk_stream_t; /* hipStream_t */
 

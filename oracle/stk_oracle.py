@@ -185,6 +185,18 @@ def activation(x, kind):
         return 0.5 * x * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
     if kind == "silu":
         return x / (1.0 + np.exp(-x))
+    # the derivatives of the four (what a backward pass multiplies the incoming gradient with)
+    if kind == "relu_grad":
+        return (x > 0.0).astype(np.float64)
+    if kind == "gelu_grad":
+        return 0.5 * (1.0 + _erf(x / math.sqrt(2.0))) + x * np.exp(-0.5 * x * x) / math.sqrt(2.0 * math.pi)
+    if kind == "gelu_tanh_grad":
+        c = math.sqrt(2.0 / math.pi)
+        t = np.tanh(c * (x + 0.044715 * x ** 3))
+        return 0.5 * (1.0 + t) + 0.5 * x * (1.0 - t * t) * c * (1.0 + 3.0 * 0.044715 * x * x)
+    if kind == "silu_grad":
+        sg = 1.0 / (1.0 + np.exp(-x))
+        return sg * (1.0 + x * (1.0 - sg))
     raise ValueError(kind)
 
 

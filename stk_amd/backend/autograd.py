@@ -213,6 +213,7 @@ class SDD(torch.autograd.Function):
                               block_offsets_t)
         ctx.shape = tuple(shape)
         out = torch.empty(data.shape, dtype=lhs.dtype, device=lhs.device)
+        backend.prepare_plan(data, offsets, column_indices, offsets_t, column_indices_t)
         backend.sdd(lhs, rhs, shape, out, offsets, row_indices, column_indices, block_order=block_offsets_t)
         return out
 
@@ -226,26 +227,24 @@ class SDD(torch.autograd.Function):
         return dlhs, drhs, None, None, None, None, None, None, None, None
 
 
-_ACTIVATION_FNS = {
-    None: lambda v: v, "none": lambda v: v, "relu": torch.relu, "silu": torch.nn.functional.silu,
-    "gelu": torch.nn.functional.gelu, "gelu_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh"),
-}
+_FUSED_ACTIVATIONS = (None, "none", "relu", "silu", "gelu", "gelu_tanh")   # (their derivatives are the backward pass's business)
 
 
 class SDDFused(torch.autograd.Function):
     """activation(sdd(lhs, rhs)) * multiplier in one pass (no counterpart in the reference, whose callers run
     the activation and stk.ops.mul, stk/ops/eltwise_ops.py:3-28, as passes of their own).  Only the result is
-    stored; backward recomputes the sums with a plain sdd, differentiates the element-wise part with torch
-    and then follows SDD.backward."""
+    stored; backward recomputes the sums in an sdd whose store applies the activation's derivative and multiplies
+    by the incoming gradient, and then follows SDD.backward."""
 
     @staticmethod
     @custom_fwd
     def forward(ctx, lhs, rhs, shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,
                 block_offsets_t, activation, multiplier):
-        if activation not in _ACTIVATION_FNS:
+        if activation not in _FUSED_ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}")
         out = torch.empty(data.shape, dtype=lhs.dtype, device=lhs.device)
         values = None if multiplier is None else multiplier.detach().contiguous()
+        backend.prepare_plan(data, offsets, column_indices, offsets_t, column_indices_t)
         backend.sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activation, values,
                           block_order=block_offsets_t)
         ctx.save_for_backward(lhs, rhs, offsets, row_indices, column_indices, offsets_t, column_indices_t,
@@ -261,18 +260,24 @@ class SDDFused(torch.autograd.Function):
         lhs, rhs, *meta = ctx.saved_tensors
         values = meta.pop() if ctx.has_multiplier else None
         offsets, row_indices, column_indices, _, _, block_offsets_t = meta
-        sums = torch.empty(dy.shape, dtype=lhs.dtype, device=lhs.device)
-        backend.sdd(lhs, rhs, ctx.shape, sums, offsets, row_indices, column_indices, block_order=block_offsets_t)
-        with torch.enable_grad():
-            pre = sums.float().requires_grad_(True)
-            act = _ACTIVATION_FNS[ctx.activation](pre)
-        g = dy.float()
+        plain = ctx.activation in (None, "none")
+        if not dy.is_contiguous():
+            dy = dy.contiguous()
+
+        def recompute(activation, multiplier):
+            out = torch.empty(dy.shape, dtype=lhs.dtype, device=lhs.device)
+            backend.sdd_fused(lhs, rhs, ctx.shape, out, offsets, row_indices, column_indices, activation, multiplier,
+                              block_order=block_offsets_t)
+            return out
+
+        # out = round(round(act(s)) * m): the gradient that reaches the sums is act'(s) * (dy * m), the one that reaches
+        # the multiplier dy * round(act(s)).  Both come out of sdd launches that compute the sums again and apply the
+        # derivative (or the activation) while they store - no element-wise passes over fp32 copies of the values.
         dmul = None
-        if values is not None:
-            if ctx.needs_input_grad[11]:
-                dmul = (g * act.detach().to(lhs.dtype).float()).to(values.dtype)   # the factor is the rounded activation
-            g = g * values.float()
-        dsums = (torch.autograd.grad(act, pre, g)[0] if act.requires_grad and act is not pre else g).to(lhs.dtype)
+        if values is not None and ctx.needs_input_grad[11]:
+            dmul = dy * recompute(ctx.activation, None)
+        g = dy if values is None else dy * values
+        dsums = g if plain else recompute(ctx.activation + "_grad", g)
         dlhs, drhs = _sdd_operand_gradients(ctx, lhs, rhs, _Sparse(ctx.shape, dsums, *meta), dsums)
         return dlhs, drhs, None, None, None, None, None, None, None, None, None, dmul
 

@@ -176,7 +176,19 @@ def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, 
     return plan
 
 
-ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3, "silu": 4}
+def prepare_plan(data, offsets, column_indices, offsets_t, column_indices_t):
+    """Builds the fusion plan of a topology for both directions if there is none yet.  sdd itself needs the block rows
+    only (its signature, the reference's, has no transpose metadata), so a plan built by its first call would be built
+    again, with the columns, by the dsd or dds that follows on the same topology; callers that have the whole metadata
+    at hand (the autograd functions) call this first and every product finds the one plan."""
+    b = data.shape[-1] if data.dim() == 3 else 0
+    if FUSION and b in (64, 128) and offsets.is_cuda and column_indices.numel() > 0:
+        fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b)
+
+
+ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3, "silu": 4,
+               # the derivatives: with the incoming gradient as the multiplier, the gradient with respect to the sums
+               "relu_grad": 5, "gelu_tanh_grad": 6, "gelu_grad": 7, "silu_grad": 8}
 
 
 def sdd(lhs, rhs, shape, out, offsets, row_indices, column_indices, block_order=None):

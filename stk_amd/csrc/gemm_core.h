@@ -88,7 +88,12 @@ __device__ __forceinline__ uint32_t mul_packed(uint32_t a, uint32_t b) {
 }
 
 // Activation functions that a product can apply to its fp32 accumulators before they are rounded.
-enum Activation : int { kNoActivation = 0, kRelu = 1, kGeluTanh = 2, kGeluErf = 3, kSilu = 4, kActivations = 5 };
+// The second four are the derivatives of the first four: with the incoming gradient as the multiplier, a sampled product
+// whose store applies one of them yields the gradient with respect to the sums of a product that applied the function.
+enum Activation : int {
+  kNoActivation = 0, kRelu = 1, kGeluTanh = 2, kGeluErf = 3, kSilu = 4,
+  kReluGrad = 5, kGeluTanhGrad = 6, kGeluErfGrad = 7, kSiluGrad = 8, kActivations = 9
+};
 template <int KIND>
 __device__ __forceinline__ float activate(float x) {
   // exp2 and the reciprocal are the hardware's approximations (1 ulp): the result is rounded to 16 bits
@@ -99,7 +104,20 @@ __device__ __forceinline__ float activate(float x) {
     return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * (k1 + k3 * x * x)));
   } else if constexpr (KIND == kGeluErf) return 0.5f * x * (1.f + erff(x * 0.7071067811865476f));
   else if constexpr (KIND == kSilu) return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
-  else return x;
+  else if constexpr (KIND == kReluGrad) return x > 0.f ? 1.f : 0.f;
+  else if constexpr (KIND == kGeluTanhGrad) {
+    // d/dx [x s], s = 1 / (1 + exp(-2 u)):  s + x s (1 - s) 2 u',  2 u' = 2 sqrt(2 / pi) (1 + 3 * 0.044715 x^2)
+    constexpr float c2 = 2.f * 0.7978845608028654f, k1 = -c2 * 1.4426950408889634f, k3 = k1 * 0.044715f;
+    const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * (k1 + k3 * x * x)));
+    return s * (1.f + x * (1.f - s) * (c2 + 3.f * 0.044715f * c2 * x * x));
+  } else if constexpr (KIND == kGeluErfGrad) {
+    // 0.5 (1 + erf(x / sqrt 2)) + x exp(-x^2 / 2) / sqrt(2 pi)
+    return 0.5f * (1.f + erff(x * 0.7071067811865476f)) + x * 0.3989422804014327f * __builtin_amdgcn_exp2f(x * x * -0.7213475204444817f);
+  } else if constexpr (KIND == kSiluGrad) {
+    // s (1 + x (1 - s)), s = 1 / (1 + exp(-x))
+    const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+    return s * (1.f + x * (1.f - s));
+  } else return x;
 }
 
 // v = activation(v) on the 16 values of an accumulator; kind is wave-uniform.
@@ -114,6 +132,10 @@ __device__ __forceinline__ void activate_all(f32x16_t& v, int kind) {
     case kGeluTanh: activate_16<kGeluTanh>(v); break;
     case kGeluErf: activate_16<kGeluErf>(v); break;
     case kSilu: activate_16<kSilu>(v); break;
+    case kReluGrad: activate_16<kReluGrad>(v); break;
+    case kGeluTanhGrad: activate_16<kGeluTanhGrad>(v); break;
+    case kGeluErfGrad: activate_16<kGeluErfGrad>(v); break;
+    case kSiluGrad: activate_16<kSiluGrad>(v); break;
     default: break;
   }
 }
@@ -631,18 +653,37 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
   const int wave = tid >> 6;
   if constexpr (Cfg::WK == 1) {
     char* s = smem + wave * 8192;  // [64 m][64 n] 16-bit, rows of 128 bytes, 8-byte units swizzled by the row
-    if (activation != kNoActivation) {
-#pragma unroll
-      for (int i = 0; i < Cfg::IM; i++)
-#pragma unroll
-        for (int j = 0; j < Cfg::JN; j++) activate_all(acc[i][j], activation);
-    }
 #pragma unroll
     for (int qi = 0; qi < (Cfg::IM + 1) / 2; qi++)
 #pragma unroll
       for (int qj = 0; qj < Cfg::JN / 2; qj++) {
         constexpr int kOdd = Cfg::IM & 1;
         const int strips = (kOdd && qi == Cfg::IM / 2) ? 1 : 2;  // 32-row strips in this pass (the last one of an odd IM has one)
+        // where piece `it` of this pass goes: row gm, eight columns from gn, element offset `at` in out (and mul)
+        auto place = [&](int it, int& gm, int& gn) {
+          const int m = it * 8 + (lane >> 3), ch = lane & 7;
+          gm = qi * 64 + m, gn = qj * 64 + ch * 8;
+          return (int64_t)gm * ldc + qj * quadrant_stride + ch * 8 + (int64_t)((row_base + gm) >> 7) * row_jump;
+        };
+        // the multiplier's values of this pass, read once: on their way while the sums are rounded and staged
+        u32x4 factor[8];
+        if (mul) {
+#pragma unroll
+          for (int it = 0; it < 8; it++) {
+            int gm, gn;
+            const int64_t at = place(it, gm, gn);
+            factor[it] = u32x4{0u, 0u, 0u, 0u};
+            if (it < 4 * strips && gm < m_valid && gn < n_valid) factor[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mul + at));
+          }
+        }
+        // (the activation of this pass's sums: arithmetic for the loads above to hide behind)
+        if (activation != kNoActivation) {
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+              if (2 * qi + i < Cfg::IM) activate_all(acc[2 * qi + i][2 * qj + j], activation);
+        }
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -664,11 +705,11 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
           int ch = lane & 7;
           u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4));
           if ((m >> 4) & 1) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
-          int gm = qi * 64 + m, gn = qj * 64 + ch * 8;
+          int gm, gn;
+          const int64_t at = place(it, gm, gn);
           if (gm < m_valid && gn < n_valid) {
-            const int64_t at = (int64_t)gm * ldc + qj * quadrant_stride + ch * 8 + (int64_t)((row_base + gm) >> 7) * row_jump;
             if (mul) {
-              const u32x4 f = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mul + at));  // read once
+              const u32x4 f = factor[it];
               v = u32x4{mul_packed<Cfg::BF16>(v.x, f.x), mul_packed<Cfg::BF16>(v.y, f.y), mul_packed<Cfg::BF16>(v.z, f.z), mul_packed<Cfg::BF16>(v.w, f.w)};
             }
             u32x4* dst = reinterpret_cast<u32x4*>(out + at);

@@ -277,7 +277,8 @@ extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_
                              int activation, const void* multiplier, stk_stream_t stream) {
   using namespace stk;
   static_assert(STK_ACT_NONE == kNoActivation && STK_ACT_RELU == kRelu && STK_ACT_GELU_TANH == kGeluTanh && STK_ACT_GELU == kGeluErf &&
-                    STK_ACT_SILU == kSilu, "the header's activation codes are the kernels'");
+                    STK_ACT_SILU == kSilu && STK_ACT_RELU_GRAD == kReluGrad && STK_ACT_GELU_TANH_GRAD == kGeluTanhGrad &&
+                    STK_ACT_GELU_GRAD == kGeluErfGrad && STK_ACT_SILU_GRAD == kSiluGrad, "the header's activation codes are the kernels'");
   if (activation < 0 || activation >= kActivations) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: activation %d", activation);
   if (multiplier && !aligned16(multiplier)) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: multiplier needs a 16-byte aligned base");
   if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: blocking %d (64 or 128)", blocking);

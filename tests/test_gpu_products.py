@@ -228,6 +228,20 @@ def test_sdd_fused_gradients(activation, with_multiplier, trans_a, trans_b):
         U.assert_close(mult.data.grad, U.np32(mf.grad), dtype, "fused grad wrt multiplier")
 
 
+@pytest.mark.parametrize("blocking,dtype", [(128, torch.bfloat16), (64, torch.float16)])
+@pytest.mark.parametrize("activation", ["relu", "gelu_tanh", "gelu", "silu"])
+def test_sdd_store_applies_the_derivative_of_an_activation(activation, blocking, dtype):
+    # the backward pass of sdd_fused in one launch: act'(lhs x rhs) * incoming gradient
+    _seed("sdd_fused_derivative", activation, blocking, dtype)
+    lhs, rhs, topo_m, g = _fused_case(384, 128, 512, 0.5, blocking, dtype)
+    from stk_amd.backend import hip_kernels
+    out = torch.empty_like(topo_m.data)
+    hip_kernels.sdd_fused(lhs, rhs, tuple(topo_m.size()), out, topo_m.offsets, topo_m.row_indices, topo_m.column_indices,
+                          activation + "_grad", g.data)
+    want = O.sdd_fused(U.np32(lhs), U.np32(rhs), U.topo_of(topo_m), activation + "_grad", U.np32(g.data))
+    U.assert_close(out, want, dtype, f"sdd with {activation}' and a multiplier")
+
+
 def test_sdd_fused_argument_contract():
     lhs, rhs, topo_m, mult = _fused_case(256, 64, 256, 0.5, 128, torch.bfloat16)
     with pytest.raises(ValueError):

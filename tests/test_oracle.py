@@ -271,6 +271,28 @@ def test_activations_against_torch_and_special_values():
         O.activation(x, "swish")
 
 
+def test_activation_derivatives_against_torch_autograd_and_differences():
+    import torch
+    import torch.nn.functional as F
+    x = np.concatenate([np.linspace(-12, 12, 4801), [1e-8, -1e-8, 30.0, -30.0]])
+    for kind, fn in (("relu", F.relu), ("gelu", F.gelu), ("gelu_tanh", lambda v: F.gelu(v, approximate="tanh")), ("silu", F.silu)):
+        pts = x[x != 0.0] if kind == "relu" else x        # (relu'(0): torch says 0, and so does the oracle; checked below)
+        t = torch.from_numpy(pts).requires_grad_(True)
+        fn(t).sum().backward()
+        got = O.activation(pts, kind + "_grad")
+        assert np.allclose(got, t.grad.numpy(), rtol=1e-10, atol=1e-12), kind
+        # central differences of the oracle's own function: a derivative of some other function would not match
+        inner = pts[(np.abs(pts) > 1e-3) & (np.abs(pts) < 11)]
+        h = 1e-6
+        diff = (O.activation(inner + h, kind) - O.activation(inner - h, kind)) / (2 * h)
+        assert np.allclose(O.activation(inner, kind + "_grad"), diff, rtol=1e-6, atol=1e-8), kind
+        # one for large positive arguments, zero for large negative ones
+        assert np.allclose(O.activation(np.array([40.0, -40.0]), kind + "_grad"), [1.0, 0.0], atol=1e-12)
+    assert O.activation(np.zeros(1), "relu_grad").tolist() == [0.0]
+    assert abs(O.activation(0.0, "gelu_grad") - 0.5) < 1e-15 and abs(O.activation(0.0, "silu_grad") - 0.5) < 1e-15
+    assert abs(O.activation(0.0, "gelu_tanh_grad") - 0.5) < 1e-15
+
+
 def test_sdd_fused_is_the_composition_of_its_parts():
     rng = np.random.RandomState(11)
     b = 16
