@@ -107,7 +107,9 @@ __device__ __forceinline__ float activate(float x) {
   else if constexpr (KIND == kReluGrad) return x > 0.f ? 1.f : 0.f;
   else if constexpr (KIND == kGeluTanhGrad) {
     // d/dx [x s], s = 1 / (1 + exp(-2 u)):  s + x s (1 - s) 2 u',  2 u' = 2 sqrt(2 / pi) (1 + 3 * 0.044715 x^2)
+    // (x is clamped: beyond +-1e4 the derivative is 1 or 0 to the last bit, and x^2 must stay finite)
     constexpr float c2 = 2.f * 0.7978845608028654f, k1 = -c2 * 1.4426950408889634f, k3 = k1 * 0.044715f;
+    x = __builtin_amdgcn_fmed3f(x, -1e4f, 1e4f);
     const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * (k1 + k3 * x * x)));
     return s * (1.f + x * (1.f - s) * (c2 + 3.f * 0.044715f * c2 * x * x));
   } else if constexpr (KIND == kGeluErfGrad) {
