@@ -76,8 +76,8 @@ __host__ __device__ inline size_t plan_list_offset(int64_t block_rows, int64_t b
 }
 // Behind the lists: per direction kPlanHintBytes bytes of hints for the launches.  Bytes 0 .. kTailSliceColumns - 1:
 // entry t = slices (1 .. kMaxTailSlices) along k for the tiles of the last round of a stk_dsd launch whose dense
-// operand has 256 (t + 1) columns (wider: as 256 * 16).  Byte kSpreadHint: 1 when the lengths of the lines drift
-// along the list, so that equal shares of the list are unequal shares of the work (see xcd_grouped()).
+// operand has 256 (t + 1) columns (wider: as 256 * 16).  Byte kSpreadHint: 1 when equal eighths of the lines hold
+// unequal numbers of blocks (read by the dsd with a sliced last round, see xcd_share()).
 constexpr int kTailSliceColumns = 16;
 constexpr int kSpreadHint = 16;
 constexpr int kPlanHintBytes = 32;
