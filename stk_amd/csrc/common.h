@@ -78,8 +78,11 @@ __host__ __device__ inline size_t plan_list_offset(int64_t block_rows, int64_t b
 // entry t = slices (1 .. kMaxTailSlices) along k for the tiles of the last round of a stk_dsd launch whose dense
 // operand has 256 (t + 1) columns (wider: as 256 * 16).  Byte kSpreadHint: 1 when equal eighths of the lines hold
 // unequal numbers of blocks (read by the dsd with a sliced last round, see xcd_share()).
+// Bytes kGroupHint .. kGroupHint + kPlanLists - 1: for each list, how many consecutive entries go to one compute die
+// at a time (see xcd_item()).
 constexpr int kTailSliceColumns = 16;
 constexpr int kSpreadHint = 16;
+constexpr int kGroupHint = 17;
 constexpr int kPlanHintBytes = 32;
 constexpr int kMaxTailSlices = 4;
 __host__ __device__ inline size_t plan_slices_offset(int64_t block_rows, int64_t block_cols) {
@@ -92,6 +95,13 @@ struct PlanLists {
   int lines;
   const uint8_t* hints;  // kPlanHintBytes of this direction
   __host__ __device__ const int32_t* list(int k) const { return lists + (int64_t)k * lines; }
+  // entries of list k that go to one compute die at a time (a wave-uniform, scalar read)
+  __device__ int group(int k) const {
+    typedef const __attribute__((address_space(4))) int32_t* words_t;
+    const int at = kGroupHint + k;
+    const int e = (((words_t)(uintptr_t)hints)[at >> 2] >> (8 * (at & 3))) & 0xff;
+    return e > 0 ? e : 1;
+  }
 };
 inline PlanLists plan_lists_of(const uint8_t* plan, int64_t block_rows, int64_t block_cols, bool columns) {
   const int32_t* base = reinterpret_cast<const int32_t*>(plan + plan_list_offset(block_rows, block_cols));

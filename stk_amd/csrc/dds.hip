@@ -59,19 +59,19 @@ __global__ __launch_bounds__(512, 2) void dds_fused64_kernel(DdsArgs g, PlanList
   int bid = blockIdx.x;
   // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles);
+    const int item = xcd_item(bid, pair_tiles, ntm, plan.group(kTallPairs));
     dds_tile<Pair, 64, TRANS_B, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntm], (item % ntm) * Pair::TM, smem, 2);
     return;
   }
   bid -= pair_tiles;
   if (bid < quad_tiles) {
-    const int item = xcd_item(bid, quad_tiles);
+    const int item = xcd_item(bid, quad_tiles, ntm, plan.group(kPairs));
     dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Quad::TM, smem, 4);
     return;
   }
   bid -= quad_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles);
+    const int item = xcd_item(bid, triple_tiles, ntm, plan.group(kTallTriples));
     dds_tile<Quad, 64, TRANS_B, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntm], (item % ntm) * Quad::TM, smem, 3);
   }
 }
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists 
   }
   const int pair_tiles = const_ints(plan.counts)[kPairs] * ntm, single_tiles = const_ints(plan.counts)[kSingles] * ntm;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles);
+    const int item = xcd_item(bid, pair_tiles, ntm, plan.group(kPairs));
     dds_tile<Fused, 128, TRANS_B, true, 2>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Fused::TM, smem);
     return;
   }

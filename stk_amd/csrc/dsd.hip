@@ -61,19 +61,19 @@ __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanList
   int bid = blockIdx.x;
   // pairs first: they hold the lines that were too long for groups of four, the longest tiles of the launch
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles);
+    const int item = xcd_item(bid, pair_tiles, ntn, plan.group(kTallPairs));
     dsd_tile<Pair, 64, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Pair::TN, smem, 2);
     return;
   }
   bid -= pair_tiles;
   if (bid < quad_tiles) {
-    const int item = xcd_item(bid, quad_tiles);
+    const int item = xcd_item(bid, quad_tiles, ntn, plan.group(kPairs));
     dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kPairs))[item / ntn], (item % ntn) * Quad::TN, smem, 4);
     return;
   }
   bid -= quad_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles);
+    const int item = xcd_item(bid, triple_tiles, ntn, plan.group(kTallTriples));
     dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntn], (item % ntn) * Quad::TN, smem, 3);
   }
 }
@@ -101,13 +101,13 @@ __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists 
   const int triple_tiles = const_ints(plan.counts)[kTallTriples] * 2 * ntn;
   const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles);
+    const int item = xcd_item(bid, pair_tiles, ntn, plan.group(kTallPairs));
     dsd_tile<Fused, 128, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
     return;
   }
   bid -= pair_tiles;
   if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles);
+    const int item = xcd_item(bid, triple_tiles, 2 * ntn, plan.group(kTallTriples));
     dsd_tile<Triple, 128, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
     return;
   }

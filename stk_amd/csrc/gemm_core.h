@@ -783,20 +783,27 @@ __device__ __forceinline__ int xcd_grouped(int bid, int n) {
   const int r = bid - base;
   return base + (r & 7) * GROUP + (r >> 3);
 }
-// Tiles of a plan's list of grouped lines (xcd_item: groups of sixteen) and the tiles of stk_sdd (xcd_tile: groups
-// of eight).  Measured against eight contiguous shares on dMoE topologies: the same or up to 6 % faster for every
-// product but the dsd with a sliced last round, which keeps the shares (xcd_share).  Equal shares of a list are
-// unequal shares of the work when the experts differ in size, and a die that lags holds the launch up.  The price
-// is operand traffic: a panel that all tiles of an expert share is fetched by every die that holds one of its
-// groups (dds on the benchmark topology: the lhs panel by four dies instead of one).  Groups of eight are another
-// 1 % faster for dds and fetch the panel eight times.
-#ifndef STK_XCD_LIST_GROUP
-#define STK_XCD_LIST_GROUP 16
-#endif
+// Tiles of a plan's list of grouped lines: `entries` consecutive list entries (with the `per` tiles of each) go to one
+// compute die at a time, eight such groups to the eight dies.  Tiles of neighbouring entries share operand panels - in a
+// dMoE topology the lines of an expert are neighbours - so a large group keeps a panel in one L2 instead of having
+// every die fetch it; but the first group of a list sorted by length is its heaviest, and once it outweighs a die's
+// fair share of the launch that die holds everything up.  The plan therefore sets `entries` per list (plan_roles_kernel:
+// a quarter of a die's share of the list's blocks, at most 32).  Measured inside a forward + backward chain of
+// products, where the operands come from memory: dds on the benchmark topology 267 -> 252 us with 32 entries instead
+// of 4, while on the Zipf-skewed top-2 topology of BASELINE's configuration 4 groups of 16 or 32 entries cost
+// 25 - 70 % (one die would get the whole of the most popular expert) and the plan picks 2 - 4 there.
+__device__ __forceinline__ int xcd_item(int bid, int n, int per, int entries) {
+  const int group = entries * per, stretch = 8 * group;
+  const int base = bid / stretch * stretch;
+  if (base + stretch > n) return bid;
+  const int r = bid - base;
+  return base + (r & 7) * group + (r >> 3);
+}
+// The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
+// to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
 #ifndef STK_XCD_SDD_GROUP
 #define STK_XCD_SDD_GROUP 8
 #endif
-__device__ __forceinline__ int xcd_item(int bid, int n) { return xcd_grouped<STK_XCD_LIST_GROUP>(bid, n); }
 __device__ __forceinline__ int xcd_tile(int bid, int n) { return xcd_grouped<STK_XCD_SDD_GROUP>(bid, n); }
 // spread (wave-uniform, a hint of the plan: the lines' lengths drift along the list): groups of kXcdGroup;
 // otherwise eight contiguous shares.

@@ -23,13 +23,13 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
     const int triple_tiles = const_ints(rows.counts)[kTallTriples] * 2 * ntn;
     const int single_tiles = const_ints(rows.counts)[kTallSingles] * ntn;
     if (bid < pair_tiles) {
-      const int item = xcd_item(bid, pair_tiles);
+      const int item = xcd_item(bid, pair_tiles, ntn, rows.group(kTallPairs));
       dsd_tile<DsdFused, 128, false, true, 2>(d, const_ints(rows.list(kTallPairs))[item / ntn], (item % ntn) * DsdFused::TN, smem);
       return;
     }
     bid -= pair_tiles;
     if (bid < triple_tiles) {
-      const int item = xcd_item(bid, triple_tiles);
+      const int item = xcd_item(bid, triple_tiles, 2 * ntn, rows.group(kTallTriples));
       dsd_tile<DsdTriple, 128, false, true, 3>(d, const_ints(rows.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * DsdTriple::TN, smem);
       return;
     }
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
   }
   const int pair_tiles = const_ints(cols.counts)[kPairs] * ntm, single_tiles = const_ints(cols.counts)[kSingles] * ntm;
   if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles);
+    const int item = xcd_item(bid, pair_tiles, ntm, cols.group(kPairs));
     dds_tile<DdsFused, 128, false, true, 2>(s, const_ints(cols.list(kPairs))[item / ntm], (item % ntm) * DdsFused::TM, smem);
     return;
   }

@@ -365,6 +365,31 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
       }
     }
     __syncthreads();
+    // How many consecutive entries of each list go to one compute die at a time (xcd_item): as many as hold a
+    // quarter of a die's share of the list's blocks when they are as long as the first, the longest, entry - the
+    // first group is the heaviest, and a die that gets too much of the launch in one piece holds it up - rounded
+    // down to a power of two, between 1 and 32.
+    for (int kind = 0; kind < kPlanLists; kind++) {
+      const int count = totals[kind];
+      const int32_t* list = lists + 2 * kPlanLists + (cols ? kPlanLists * block_rows : 0) + kind * lines;
+      int mine_blocks = 0;
+      for (int e = tid; e < count; e += 1024) {
+        const int line = list[e];
+        mine_blocks += offs[line + 1] - offs[line];
+      }
+      int total_blocks;
+      block_exclusive_scan(mine_blocks, wave_last, &total_blocks);
+      if (tid == 0) {
+        int entries = 1;
+        if (count > 0) {
+          const int first = list[0], longest = offs[first + 1] - offs[first];
+          const int fit = total_blocks / (32 * (longest > 0 ? longest : 1));
+          while (entries < 32 && 2 * entries <= fit) entries *= 2;
+        }
+        tail_slices[kGroupHint + kind] = (uint8_t)entries;
+      }
+    }
+    __syncthreads();
   }
   // Tiles of stk_sdd (block rows only), row by row: groups of identical rows (sdd_rows_owned) times up to
   // sdd_cols neighbouring blocks (one for a group of three rows).

@@ -258,6 +258,19 @@ def test_fusion_plan_roles(name):
         assert all(1 <= int(v) <= 4 for v in h[:16])
         shares = [int(offs[(c + 1) * lines // 8]) - int(offs[c * lines // 8]) for c in range(8)]
         assert int(h[16]) == int(any(32 * sh > 5 * int(offs[lines]) for sh in shares)), (d, shares)
+        # and per list the entries that go to one compute die at a time: a quarter of a die's share of the list's
+        # blocks in entries as long as the first one, rounded down to a power of two between 1 and 32
+        base = 10 + (5 * br if d else 0)
+        for kind in range(5):
+            count = int(lists[5 * d + kind])
+            entries = 1
+            if count:
+                members = lists[base + kind * lines: base + kind * lines + count].tolist()
+                blocks = [int(offs[i + 1]) - int(offs[i]) for i in members]
+                fit = sum(blocks) // (32 * max(blocks[0], 1))
+                while entries < 32 and 2 * entries <= fit:
+                    entries *= 2
+            assert int(h[17 + kind]) == entries, (d, kind, count)
     # in front: the tiles of sdd
     sdd = whole[:8 + 8 * max_tiles].view(np.int32)
     assert sdd[2:2 + 2 * sdd[0]].reshape(-1, 2).tolist() == _sdd_tiles(topo.offsets, topo.column_indices, 2, 2)
