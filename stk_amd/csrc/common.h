@@ -76,9 +76,12 @@ __host__ __device__ inline size_t plan_list_offset(int64_t block_rows, int64_t b
 }
 // Behind the lists: per direction kPlanHintBytes bytes of hints for the launches.  Bytes 0 .. kTailSliceColumns - 1:
 // entry t = slices (1 .. kMaxTailSlices) along k for the tiles of the last round of a stk_dsd launch whose dense
-// operand has 256 (t + 1) columns (wider: as 256 * 16).  Bytes kGroupHint .. kGroupHint + kPlanLists - 1: for each
-// list, how many consecutive entries go to one compute die at a time (see xcd_item()).  The rest is zero.
+// operand has 256 (t + 1) columns (wider: as 256 * 16).  Byte kSpreadHint: 1 when equal eighths of the lines hold
+// unequal numbers of blocks (read by the dsd with a sliced last round, see xcd_share()).
+// Bytes kGroupHint .. kGroupHint + kPlanLists - 1: for each list, how many consecutive entries go to one compute die
+// at a time (see xcd_item()).
 constexpr int kTailSliceColumns = 16;
+constexpr int kSpreadHint = 16;
 constexpr int kGroupHint = 17;
 constexpr int kPlanHintBytes = 32;
 constexpr int kMaxTailSlices = 4;

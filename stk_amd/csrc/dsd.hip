@@ -255,6 +255,7 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
   const int tiles = pair_tiles + triple_tiles + single_tiles;
   int slices = uniform(plan.hints[(ntn < kTailSliceColumns ? ntn : kTailSliceColumns) - 1]);
+  const bool spread = (const_ints(plan.hints)[kSpreadHint / 4] & 0xff) != 0;
   if (slices < 1 || slices > kMaxTailSlices) slices = 1;
   // whole rounds first; the rest (all of it when there is less than one round) is the last round
   int whole = (slices > 1 && tiles > 0) ? (tiles - 1) / t.workgroups * t.workgroups : tiles;
@@ -276,13 +277,13 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   }
   const int ordinal = item - whole;  // among the tiles of the last round: 0 .. workgroups - 1
   if (item < pair_tiles) {
-    const int i = xcd_item(item, pair_tiles, ntn, plan.group(kTallPairs));
+    const int i = xcd_share(item, pair_tiles, spread);
     dsd_slice<Fused, TRANS_A, 2>(g, t, const_ints(plan.list(kTallPairs))[i / ntn], (i % ntn) * Fused::TN, slice, slices, ordinal, smem, &flag);
     return;
   }
   item -= pair_tiles;
   if (item < triple_tiles) {
-    const int i = xcd_item(item, triple_tiles, 2 * ntn, plan.group(kTallTriples));
+    const int i = xcd_share(item, triple_tiles, spread);
     dsd_slice<Triple, TRANS_A, 3>(g, t, const_ints(plan.list(kTallTriples))[i / (2 * ntn)], (i % (2 * ntn)) * Triple::TN, slice, slices, ordinal, smem, &flag);
     return;
   }

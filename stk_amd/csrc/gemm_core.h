@@ -800,10 +800,13 @@ __device__ __forceinline__ int xcd_item(int bid, int n, int per, int entries) {
   return base + (r & 7) * group + (r >> 3);
 }
 // The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
-// to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size); the same for
-// the dsd with a sliced last round once it was timed inside a chain of products instead of back to back.
+// to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
 #ifndef STK_XCD_SDD_GROUP
 #define STK_XCD_SDD_GROUP 8
 #endif
 __device__ __forceinline__ int xcd_tile(int bid, int n) { return xcd_grouped<STK_XCD_SDD_GROUP>(bid, n); }
+// spread (wave-uniform, a hint of the plan: the lines' lengths drift along the list): groups of kXcdGroup;
+// otherwise eight contiguous shares.
+__device__ __forceinline__ int xcd_share(int bid, int n, bool spread) { return spread ? xcd_grouped(bid, n) : xcd_chunked(bid, n); }
+
 }  // namespace stk

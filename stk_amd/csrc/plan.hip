@@ -389,8 +389,6 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
         tail_slices[kGroupHint + kind] = (uint8_t)entries;
       }
     }
-    // (the bytes of the hints that nothing uses)
-    if (tid >= kTailSliceColumns && tid < kPlanHintBytes && (tid < kGroupHint || tid >= kGroupHint + kPlanLists)) tail_slices[tid] = 0;
     __syncthreads();
   }
   // Tiles of stk_sdd (block rows only), row by row: groups of identical rows (sdd_rows_owned) times up to
@@ -447,6 +445,20 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
 #pragma unroll
     for (int k = 0; k < kMaxTailSlices; k++) ends[k] = __shfl(end, (tid & ~3) + k, 64);
     if (tid % kMaxTailSlices == 0) tail_slices[tid / kMaxTailSlices] = (uint8_t)choose_tail_slices(ends);
+  }
+  // Do equal eighths of the lines hold about equal numbers of blocks?  If not (one share 25 % above the mean),
+  // the products spread the list over the XCDs in small groups instead of eight contiguous shares.
+  if (tid == 64) {
+    const int32_t* offs = cols ? offsets_t : offsets;
+    int spread = 0;
+    if (offs) {
+      const int64_t total = offs[lines];
+      for (int c = 0; c < 8; c++) {
+        const int64_t share = offs[(int64_t)(c + 1) * lines / 8] - offs[(int64_t)c * lines / 8];
+        if (share * 32 > total * 5) spread = 1;  // > 1.25 / 8 of the blocks
+      }
+    }
+    tail_slices[kSpreadHint] = (uint8_t)spread;
   }
 }
 

@@ -250,12 +250,14 @@ def test_fusion_plan_roles(name):
             expect = _longest_first(expect, offs)   # every list: longest first, equal lengths in ascending order
             assert int(lists[5 * d + kind]) == len(expect)
             assert lists[base + kind * lines: base + kind * lines + len(expect)].tolist() == expect
-    # behind the lists, per direction: slice counts for dsd (1 .. 4), an unused byte,
+    # behind the lists, per direction: slice counts for dsd (1 .. 4) and the hint that the blocks are spread
+    # unevenly over equal eighths of the lines
     hints = got[off + 4 * 5 * (2 + br + bc):]
     for d, (lines, offs) in enumerate([(br, topo.offsets), (bc, topo.offsets_t)]):
         h = hints[32 * d:32 * d + 32]
         assert all(1 <= int(v) <= 4 for v in h[:16])
-        assert int(h[16]) == 0 and not h[22:32].any()
+        shares = [int(offs[(c + 1) * lines // 8]) - int(offs[c * lines // 8]) for c in range(8)]
+        assert int(h[16]) == int(any(32 * sh > 5 * int(offs[lines]) for sh in shares)), (d, shares)
         # and per list the entries that go to one compute die at a time: a quarter of a die's share of the list's
         # blocks in entries as long as the first one, rounded down to a power of two between 1 and 32
         base = 10 + (5 * br if d else 0)
