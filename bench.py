@@ -506,7 +506,10 @@ def main():
         # untimed: the step itself until the clocks have settled; the comparators then run at the same clocks
         preheat_steps = preheat(args.preheat_ms)
         dense = dense_comparators(rows, dev, aux_steps, 5)
-        routing = routing_times(dev, aux_steps, 5)
+        try:
+            routing = routing_times(dev, aux_steps, 5)
+        except Exception as exc:  # noqa: BLE001  (auxiliary: see other_configs below)
+            routing = {"error": f"{type(exc).__name__}: {exc}"[:300]}
         preheat_steps += preheat(args.preheat_ms / 3)
         for _ in range(args.warmup):
             step()
@@ -527,12 +530,19 @@ def main():
         per_op_ms = {n: float(np.mean([e[i].elapsed_time(e[i + 1]) for e in evs])) for i, n in enumerate(names)}
         # and each product on its own, back to back
         per_op_b2b_ms = {n: time_batch(product, args.steps) for n, product in zip(names, products)}
-        gradient_pair = gradient_pair_times(topo, x, w1, args.steps)
+        try:
+            gradient_pair = gradient_pair_times(topo, x, w1, args.steps)
+        except Exception as exc:  # noqa: BLE001
+            gradient_pair = {"error": f"{type(exc).__name__}: {exc}"[:300]}
         gc.enable()
 
         others = {}
         for name in extra:
-            others[name] = other_config(name, dev, max(5, args.steps // 2), 3)
+            # (an auxiliary measurement that fails - out of memory on a busy box, say - must not take the line with it)
+            try:
+                others[name] = other_config(name, dev, max(5, args.steps // 2), 3)
+            except Exception as exc:  # noqa: BLE001
+                others[name] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
             torch.cuda.empty_cache()
 
     ms_per_step = wall * 1e3 / args.steps
@@ -587,7 +597,10 @@ def main():
     if others:
         result["other_configs"] = others
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(tokens_per_expert)
+        try:
+            result["cpu_baseline"] = cpu_baseline(tokens_per_expert)
+        except Exception as exc:  # noqa: BLE001  (the line with the GPU figures is worth more than no line)
+            result["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     print(json.dumps(result))
 
 
