@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 11
+#define STK_AMD_ABI_VERSION 12
 
 /* status codes */
 #define STK_OK 0
@@ -231,6 +231,28 @@ int stk_dsd_dds(int64_t m, int64_t k,
                 const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
                 int64_t n_dsd, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, void* out_dsd, int64_t out_dsd_stride,
                 int64_t m_dds, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k, void* out_dds, int64_t out_dds_stride,
+                int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
+
+/*
+ * Both gradients of y = op(S) * rhs in one call.  With the incoming gradient dy and S's topology [m, n],
+ *   out_sdd (nnz blocks) = lhs [m, k_sdd] * rhs_sdd [k_sdd, n] on the topology   the gradient with respect to S's values
+ *   out_dsd [.., n_dsd]  = op(S) * rhs_dsd [.., n_dsd], S's values in `data`     the gradient with respect to rhs
+ * where for op(S) = S the caller passes lhs = dy, rhs_sdd = rhs^T, transpose_a = 1 and rhs_dsd = dy, and for
+ * op(S) = S^T lhs = rhs, rhs_sdd = dy^T, transpose_a = 0 and rhs_dsd = dy.  Replaces the pair of backend calls in
+ * DSD.backward, stk/backend/sputnik.py:131-155 (sdd at :139-145, dsd at :146-154), which are two launches.  With
+ * blocking 128, a plan, more nonzero blocks than compute units, a row-major lhs and rhs_sdd as a .t() view of a
+ * row-major [n, k_sdd] with k_sdd a multiple of 64, and a row-major rhs_dsd with n_dsd a multiple of 256, both
+ * products run as one grid: the tiles of the sdd first, the tiles of the dsd behind them.  Any other case runs stk_sdd
+ * and then stk_dsd (without a workspace).  Either way the results are those of stk_sdd and of stk_dsd without a
+ * workspace, bit for bit.  Arguments as for stk_sdd (block_order = block_offsets_t) and stk_dsd.
+ */
+int stk_sdd_dsd(int64_t m, int64_t n,
+                const int32_t* offsets, const void* row_indices, const void* column_indices,
+                const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                const void* rhs_sdd, int64_t rhs_sdd_stride_k, int64_t rhs_sdd_stride_n, int64_t k_sdd, void* out_sdd,
+                const void* data, int transpose_a, int64_t n_dsd, const void* rhs_dsd, int64_t rhs_dsd_stride_k, int64_t rhs_dsd_stride_n,
+                void* out_dsd, int64_t out_dsd_stride,
                 int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
 
 /*

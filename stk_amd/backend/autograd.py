@@ -68,6 +68,9 @@ def _run_sdd(lhs, rhs, sp):
 # fill the compute units that the other leaves idle in its last round.
 OVERLAP_GRADIENTS = True
 _side_streams = {}
+# Both gradients of sdd (stk_dsd_dds) and of dsd (stk_sdd_dsd) in one launch each where the operands' layouts allow it,
+# instead of two launches side by side; the same results.
+JOINT_GRADIENTS = True
 
 
 def _side_stream(device):
@@ -118,6 +121,16 @@ class DSD(torch.autograd.Function):
         dy = _plain(dy)
         want_data = want_rhs = None
         rhs_is_view = _is_transposed_view(rhs)
+        if JOINT_GRADIENTS and ctx.needs_input_grad[1] and ctx.needs_input_grad[9] and not rhs_is_view:
+            # dy rhs^T on the pattern and op(S)^T dy read the same dy: one call (sputnik.py:131-155 makes two)
+            ddata = torch.empty_like(data)
+            drhs = torch.empty_like(rhs, memory_format=torch.contiguous_format)
+            backend.prepare_plan(data, meta[0], meta[2], meta[3], meta[4])
+            if ta:
+                backend.sdd_dsd(sp.shape, rhs, dy.t(), ddata, data, *meta, False, dy, drhs)
+            else:
+                backend.sdd_dsd(sp.shape, dy, rhs.t(), ddata, data, *meta, True, dy, drhs)
+            return None, ddata, None, None, None, None, None, None, None, drhs
         if ctx.needs_input_grad[1]:
             # d op(S) = dy rhs^T on the pattern; for a transposed S the stored blocks hold (rhs dy^T)
             want_data = (lambda: _run_sdd(rhs, dy.t(), sp)) if ta else (lambda: _run_sdd(dy, rhs.t(), sp))
@@ -168,11 +181,6 @@ class DDS(torch.autograd.Function):
         if dlhs is not None and lhs_is_view:
             dlhs = dlhs.t()
         return dlhs, None, ddata, None, None, None, None, None, None, None
-
-
-# Both gradients of sdd in one launch (stk_dsd_dds) where the operands' layouts allow it, instead of two launches
-# side by side; the same results.
-JOINT_GRADIENTS = True
 
 
 def _sdd_operand_gradients(ctx, lhs, rhs, sp, ds):

@@ -360,6 +360,36 @@ def dsd_dds(shape, data, offsets, row_indices, column_indices, offsets_t, column
             data.shape[0], b, _value_dtype(data), _INDEX_DTYPES[ci.dtype], plan.data_ptr() if plan is not None else None, _stream()))
 
 
+def sdd_dsd(shape, lhs, rhs_sdd, out_sdd, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t,
+            transpose_a, rhs_dsd, out_dsd):
+    """out_sdd = lhs @ rhs_sdd on the topology [m, n] = `shape` and out_dsd = op(sparse) @ rhs_dsd for the values `data` on the
+    same topology, in one launch where the layouts allow it (the two gradients of dsd, stk/backend/sputnik.py:131-155);
+    otherwise the two products one after the other.  The results are those of sdd and dsd (without its workspace), bit
+    for bit."""
+    _need_gpu(data, lhs, rhs_sdd, rhs_dsd, out_sdd, out_dsd)
+    m, n = shape
+    b = _blocking(data)
+    assert lhs.shape[0] == m and rhs_sdd.shape[1] == n and lhs.shape[1] == rhs_sdd.shape[0], "incompatible dimensions"
+    assert rhs_dsd.shape[0] == (m if transpose_a else n), "incompatible dimensions"
+    _validate_matmul_dims(m, lhs.shape[1], n, b)
+    _validate_matmul_dims(n if transpose_a else m, rhs_dsd.shape[0], rhs_dsd.shape[1], b)
+    lhs, rhs_sdd, rhs_dsd = _dense_operand(lhs), _dense_operand(rhs_sdd), _dense_operand(rhs_dsd)
+    data = data.detach()
+    assert data.is_contiguous() and out_sdd.is_contiguous() and out_sdd.shape == data.shape and out_dsd.stride(1) == 1
+    assert data.dtype == lhs.dtype == rhs_sdd.dtype == rhs_dsd.dtype == out_sdd.dtype == out_dsd.dtype
+    ri, ci, cit = _index(row_indices), _index(column_indices), _index(column_indices_t)
+    assert ri.dtype == ci.dtype == cit.dtype
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b) if FUSION and b in (64, 128) and data.shape[0] > 0 else None
+    with _on_device(out_dsd.device):
+        _lib.check(_lib.load().stk_sdd_dsd(
+            m, n, _offsets(offsets).data_ptr(), ri.data_ptr(), ci.data_ptr(),
+            _offsets(offsets_t).data_ptr(), cit.data_ptr(), _offsets(block_offsets_t).data_ptr(),
+            lhs.data_ptr(), lhs.stride(0), lhs.stride(1), rhs_sdd.data_ptr(), rhs_sdd.stride(0), rhs_sdd.stride(1), lhs.shape[1],
+            out_sdd.data_ptr(), data.data_ptr(), 1 if transpose_a else 0, rhs_dsd.shape[1], rhs_dsd.data_ptr(), rhs_dsd.stride(0),
+            rhs_dsd.stride(1), out_dsd.data_ptr(), out_dsd.stride(0),
+            data.shape[0], b, _value_dtype(data), _INDEX_DTYPES[ci.dtype], plan.data_ptr() if plan is not None else None, _stream()))
+
+
 def row_indices(shape, data, offsets, column_indices, out):
     """out[offsets[r]:offsets[r+1]] = r for every block row r."""
     _need_gpu(offsets, out)

@@ -78,44 +78,20 @@ __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanList
   }
 }
 
-// 128-blocks, eight wavefronts.  The workgroups take their tiles from the lists of the plan,
-// the large ones first:
-//   pairs of identical rows   256x256 tiles
-//   three identical rows      384x128 tiles: the dense operand, the big stream when rows
-//                             are long, is still read only once for the three
-//   lone rows                 128x256 tiles
+// 128-blocks, eight wavefronts.  The workgroups take their tiles from the lists of the plan (dsd_plan_tile).
 // Covered rows get no workgroup; the grid is an upper bound and the surplus leaves at once.
 // Without a plan every row is a lone row.
 template <class Fused, class Triple, class Single, bool TRANS_A>
 __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists plan) {
   extern __shared__ __align__(16) char smem[];
-  static_assert(Fused::TN == Single::TN && Fused::TN == 2 * Triple::TN, "same column tiling");
-  const int ntn = g.n / Fused::TN;
   int bid = blockIdx.x;
   if (!plan.counts) {
+    const int ntn = g.n / Fused::TN;
     const int item = xcd_grouped(bid, g.block_rows * ntn);
     dsd_tile<Single, 128, TRANS_A, true, 1>(g, item / ntn, (item % ntn) * Single::TN, smem);
     return;
   }
-  const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
-  const int triple_tiles = const_ints(plan.counts)[kTallTriples] * 2 * ntn;
-  const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
-  if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, ntn, plan.group(kTallPairs));
-    dsd_tile<Fused, 128, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
-    return;
-  }
-  bid -= pair_tiles;
-  if (bid < triple_tiles) {
-    const int item = xcd_item(bid, triple_tiles, 2 * ntn, plan.group(kTallTriples));
-    dsd_tile<Triple, 128, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
-    return;
-  }
-  bid -= triple_tiles;
-  if (bid < single_tiles) {
-    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
-    dsd_tile<Single, 128, TRANS_A, true, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
-  }
+  dsd_plan_tile<Fused, Triple, Single, TRANS_A>(g, plan, bid, smem);
 }
 
 // ---------------------------------------------------------------------------

@@ -1,5 +1,5 @@
-// Tile functions of stk_dsd, shared by its kernels (dsd.hip) and by the launch that computes a dsd and a dds on
-// the same sparse operand together (grad.hip).
+// Tile functions of stk_dsd, shared by its kernels (dsd.hip) and by the launches that compute a dsd together with
+// another product on the same topology (grad.hip).
 #pragma once
 #include "common.h"
 #include "gemm_core.h"
@@ -93,6 +93,41 @@ __device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char*
   f32x16_t acc[Cfg::IM][Cfg::JN] = {};
   dsd_accumulate<Cfg, BLK, TRANS_A, FULL, LINES>(acc, g, bi, n0, 0, g.walk_offsets[bi + 1] - g.walk_offsets[bi], smem, lines);
   dsd_store<Cfg, BLK>(acc, g, bi, n0, smem, lines * BLK);
+}
+
+// The tile of a launch over the plan's lists of lines (128-blocks, eight wavefronts) that workgroup `bid` takes,
+// the large ones first:
+//   pairs of identical rows   256x256 tiles
+//   three identical rows      384x128 tiles: the dense operand, the big stream when rows
+//                             are long, is still read only once for the three
+//   lone rows                 128x256 tiles
+// False when the lists have fewer tiles than that; bid then counts on past them.
+template <class Fused, class Triple, class Single, bool TRANS_A>
+__device__ __forceinline__ bool dsd_plan_tile(const DsdArgs& g, const PlanLists& plan, int& bid, char* smem) {
+  static_assert(Fused::TN == Single::TN && Fused::TN == 2 * Triple::TN, "same column tiling");
+  const int ntn = g.n / Fused::TN;
+  const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
+  const int triple_tiles = const_ints(plan.counts)[kTallTriples] * 2 * ntn;
+  const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
+  if (bid < pair_tiles) {
+    const int item = xcd_item(bid, pair_tiles, ntn, plan.group(kTallPairs));
+    dsd_tile<Fused, 128, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
+    return true;
+  }
+  bid -= pair_tiles;
+  if (bid < triple_tiles) {
+    const int item = xcd_item(bid, triple_tiles, 2 * ntn, plan.group(kTallTriples));
+    dsd_tile<Triple, 128, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
+    return true;
+  }
+  bid -= triple_tiles;
+  if (bid < single_tiles) {
+    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
+    dsd_tile<Single, 128, TRANS_A, true, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
+    return true;
+  }
+  bid -= single_tiles;
+  return false;
 }
 
 }  // namespace stk

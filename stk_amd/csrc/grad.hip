@@ -1,4 +1,4 @@
-// stk_dsd_dds: the two operand gradients of a sampled product in one launch.
+// stk_dsd_dds and stk_sdd_dsd: the two gradients of a product in one launch.
 //
 // The backward pass of S = lhs x rhs (sampled on a topology) computes dS x rhs^T, a dsd, and lhs^T x dS, a dds,
 // from the same sparse values dS.  Here both run as one grid: first the tiles of the dsd (long walks along a block
@@ -6,8 +6,14 @@
 // units that the last long ones leave idle, and the blocks of dS that the dsd brought into the caches are still
 // on their way through them when the dds asks for them.  The tiles are the ones of stk_dsd and stk_dds
 // (dsd_tile.h, dds_tile.h), so the results are theirs bit for bit.
+//
+// The backward pass of y = op(S) x rhs computes dy x rhs^T on the topology, an sdd, and op(S)^T x dy, a dsd, from
+// the same dy.  stk_sdd_dsd runs them as one grid in the same way: the tiles of the sdd, which contract over all
+// of rhs's columns, then the tiles of the dsd (sdd_tile.h, dsd_tile.h).
 #include "dds_tile.h"
 #include "dsd_tile.h"
+#include "sdd_tile.h"
+#include <initializer_list>
 
 namespace stk {
 
@@ -15,32 +21,10 @@ namespace stk {
 template <class DsdFused, class DsdTriple, class DsdSingle, class DdsFused, class DdsSingle>
 __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists rows, DdsArgs s, PlanLists cols) {
   extern __shared__ __align__(16) char smem[];
-  static_assert(DsdFused::TN == DsdSingle::TN && DsdFused::TN == 2 * DsdTriple::TN && DdsFused::TM == DdsSingle::TM, "same tiling");
-  const int ntn = d.n / DsdFused::TN, ntm = s.m / DdsFused::TM;
+  static_assert(DdsFused::TM == DdsSingle::TM, "same row tiling");
+  const int ntm = s.m / DdsFused::TM;
   int bid = blockIdx.x;
-  {
-    const int pair_tiles = const_ints(rows.counts)[kTallPairs] * ntn;
-    const int triple_tiles = const_ints(rows.counts)[kTallTriples] * 2 * ntn;
-    const int single_tiles = const_ints(rows.counts)[kTallSingles] * ntn;
-    if (bid < pair_tiles) {
-      const int item = xcd_item(bid, pair_tiles, ntn, rows.group(kTallPairs));
-      dsd_tile<DsdFused, 128, false, true, 2>(d, const_ints(rows.list(kTallPairs))[item / ntn], (item % ntn) * DsdFused::TN, smem);
-      return;
-    }
-    bid -= pair_tiles;
-    if (bid < triple_tiles) {
-      const int item = xcd_item(bid, triple_tiles, 2 * ntn, rows.group(kTallTriples));
-      dsd_tile<DsdTriple, 128, false, true, 3>(d, const_ints(rows.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * DsdTriple::TN, smem);
-      return;
-    }
-    bid -= triple_tiles;
-    if (bid < single_tiles) {
-      const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
-      dsd_tile<DsdSingle, 128, false, true, 1>(d, const_ints(rows.list(kTallSingles))[item / ntn], (item % ntn) * DsdSingle::TN, smem);
-      return;
-    }
-    bid -= single_tiles;
-  }
+  if (dsd_plan_tile<DsdFused, DsdTriple, DsdSingle, false>(d, rows, bid, smem)) return;
   const int pair_tiles = const_ints(cols.counts)[kPairs] * ntm, single_tiles = const_ints(cols.counts)[kSingles] * ntm;
   if (bid < pair_tiles) {
     const int item = xcd_item(bid, pair_tiles, ntm, cols.group(kPairs));
@@ -54,9 +38,9 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
   }
 }
 
-constexpr int largest(int a, int b, int c, int d, int e) {
-  int most = a;
-  for (int v : {b, c, d, e}) most = v > most ? v : most;
+constexpr int largest(std::initializer_list<int> values) {
+  int most = 0;
+  for (int v : values) most = v > most ? v : most;
   return most;
 }
 
@@ -70,13 +54,50 @@ static void launch_dsd_dds(const DsdArgs& d, const PlanLists& rows, const DdsArg
   using DsdTriple = TileCfg<4, 2, 3, 2, 1, 3, 1, true, true, BF16, 64, 2>;
   using DdsFused = TileCfg<4, 2, 2, 4, 1, 2, 2, false, false, BF16, STK_DDS_KT, STK_DDS_STAGES, STREAM>;
   using DdsSingle = TileCfg<4, 2, 2, 2, 1, 2, 1, false, false, BF16, STK_DDS_KT, STK_DDS_STAGES, STREAM>;
-  constexpr int lds = largest(DsdFused::kSmemBytes, DsdSingle::kSmemBytes, DsdTriple::kSmemBytes, DdsFused::kSmemBytes, DdsSingle::kSmemBytes);
+  constexpr int lds = largest({DsdFused::kSmemBytes, DsdSingle::kSmemBytes, DsdTriple::kSmemBytes, DdsFused::kSmemBytes, DdsSingle::kSmemBytes});
   auto kernel = &dsd_dds_kernel<DsdFused, DsdTriple, DsdSingle, DdsFused, DdsSingle>;
   static const int once = (set_lds_limit(kernel, lds), 0);
   (void)once;
   // upper bound: every line a tile of its own in both products
   const int grid = d.block_rows * (d.n / DsdFused::TN) + s.block_cols * (s.m / DdsFused::TM);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, d, rows, s, cols);
+}
+
+// 128-blocks, eight wavefronts: the tiles of the sdd from the plan's tile list as in sdd_fused_kernel, then the tiles
+// of the dsd from the plan's lists of lines as in dsd_fused_kernel.  The grid is an upper bound for both.
+template <class SddQuad, class SddPair, class SddTriple, class DsdFused, class DsdTriple, class DsdSingle, bool TRANS_A>
+__global__ __launch_bounds__(512, 2) void sdd_dsd_kernel(SddArgs a, DsdArgs d, PlanLists lines) {
+  extern __shared__ __align__(16) char smem[];
+  const int count = const_ints(a.tiles)[0];
+  int bid = blockIdx.x;
+  if (bid < count) {
+    sdd_plan_tile<SddQuad, SddPair, SddTriple, true>(a, xcd_tile(bid, count), smem);
+    return;
+  }
+  bid -= count;
+  dsd_plan_tile<DsdFused, DsdTriple, DsdSingle, TRANS_A>(d, lines, bid, smem);
+}
+
+// Both operands of the sdd K-major (a row-major lhs and a .t() view as rhs), rhs of the dsd row-major: the layouts the
+// backward pass of a product with a row-major rhs produces.  STREAM: the rhs panels of the dsd are read about once.
+template <bool BF16, bool TRANS_A, bool STREAM>
+static void launch_sdd_dsd(const SddArgs& a, const DsdArgs& d, const PlanLists& lines, hipStream_t stream) {
+  // the configurations of launch_sdd (both operands K-major: 64-deep K-tiles on two stages) and launch_dsd
+  using SddQuad = TileCfg<4, 2, 2, 4, 1, 2, 2, true, true, BF16, 64, 2>;
+  using SddPair = TileCfg<2, 4, 2, 2, 1, 1, 2, true, true, BF16, 64, 2>;
+  using SddTriple = TileCfg<4, 2, 3, 2, 1, 3, 1, true, true, BF16, 64, 2>;
+  constexpr int KT = TRANS_A ? STK_DSD_T_KT : STK_DSD_KT, S = TRANS_A ? STK_DSD_T_STAGES : STK_DSD_STAGES;
+  using DsdFused = TileCfg<4, 2, 2, 4, 1, 2, 2, !TRANS_A, false, BF16, KT, S, false, STREAM>;
+  using DsdSingle = TileCfg<2, 4, 2, 2, 1, 1, 2, !TRANS_A, false, BF16, KT, S, false, STREAM>;
+  using DsdTriple = TileCfg<4, 2, 3, 2, 1, 3, 1, !TRANS_A, false, BF16, KT, S, false, STREAM>;
+  constexpr int lds = largest({SddQuad::kSmemBytes, SddPair::kSmemBytes, SddTriple::kSmemBytes, DsdFused::kSmemBytes, DsdSingle::kSmemBytes,
+                               DsdTriple::kSmemBytes});
+  auto kernel = &sdd_dsd_kernel<SddQuad, SddPair, SddTriple, DsdFused, DsdTriple, DsdSingle, TRANS_A>;
+  static const int once = (set_lds_limit(kernel, lds), 0);
+  (void)once;
+  // upper bound: the tile list of the sdd at its longest, every line of the dsd a tile of its own
+  const int grid = (int)sdd_max_tiles(a.block_rows, a.nnz) + d.block_rows * (d.n / DsdFused::TN);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, a, d, lines);
 }
 
 }  // namespace stk
@@ -115,4 +136,44 @@ extern "C" int stk_dsd_dds(int64_t m, int64_t k,
     else launch_dsd_dds<false, false>(dsd.g, dsd.lists, dds.g, dds.lists, s);
   }
   return check_launch("stk_dsd_dds");
+}
+
+extern "C" int stk_sdd_dsd(int64_t m, int64_t n,
+                           const int32_t* offsets, const void* row_indices, const void* column_indices,
+                           const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                           const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                           const void* rhs_sdd, int64_t rhs_sdd_stride_k, int64_t rhs_sdd_stride_n, int64_t k_sdd, void* out_sdd,
+                           const void* data, int transpose_a, int64_t n_dsd, const void* rhs_dsd, int64_t rhs_dsd_stride_k, int64_t rhs_dsd_stride_n,
+                           void* out_dsd, int64_t out_dsd_stride,
+                           int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
+  using namespace stk;
+  SddProblem sdd;
+  DsdProblem dsd;
+  int rc = sdd_problem("stk_sdd_dsd", lhs, lhs_stride_m, lhs_stride_k, rhs_sdd, rhs_sdd_stride_k, rhs_sdd_stride_n, m, k_sdd, n, out_sdd, offsets,
+                       row_indices, column_indices, block_offsets_t, nnz, blocking, dtype, index_dtype, plan, STK_ACT_NONE, nullptr, &sdd);
+  if (rc != STK_OK) return rc;
+  // the dsd multiplies op(S): [m, n] as stored, [n, m] transposed
+  const int64_t m_dsd = transpose_a ? n : m, k_dsd = transpose_a ? m : n;
+  rc = dsd_problem("stk_sdd_dsd", m_dsd, k_dsd, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, transpose_a,
+                   rhs_dsd, rhs_dsd_stride_k, rhs_dsd_stride_n, out_dsd, out_dsd_stride, nnz, blocking, dtype, index_dtype, plan, &dsd);
+  if (rc != STK_OK) return rc;
+  const bool together = plan && blocking == 128 && !sdd.empty && !dsd.empty && sdd.g.tiles && nnz > compute_units() && sdd.ak && sdd.bk &&
+                        k_sdd % 64 == 0 && !dsd.bk && n_dsd % 256 == 0 && !dsd.g.small;
+  if (!together) {
+    // shapes or layouts the joint launch has no tiles for: the two products one after the other
+    rc = stk_sdd(lhs, lhs_stride_m, lhs_stride_k, rhs_sdd, rhs_sdd_stride_k, rhs_sdd_stride_n, m, k_sdd, n, out_sdd, offsets, row_indices,
+                 column_indices, block_offsets_t, nnz, blocking, dtype, index_dtype, plan, stream);
+    if (rc != STK_OK) return rc;
+    return stk_dsd(m_dsd, k_dsd, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, transpose_a, rhs_dsd,
+                   rhs_dsd_stride_k, rhs_dsd_stride_n, out_dsd, out_dsd_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define STK_SDD_DSD_CASE(BF, TA)                                                                   \
+  if ((dtype == STK_BF16) == BF && dsd.ta == TA) {                                                 \
+    if (dsd.stream_rhs) launch_sdd_dsd<BF, TA, true>(sdd.g, dsd.g, dsd.lists, s);                  \
+    else launch_sdd_dsd<BF, TA, false>(sdd.g, dsd.g, dsd.lists, s);                                \
+    return check_launch("stk_sdd_dsd");                                                            \
+  }
+  STK_SDD_DSD_CASE(true, true) STK_SDD_DSD_CASE(true, false) STK_SDD_DSD_CASE(false, true) STK_SDD_DSD_CASE(false, false)
+  return fail(STK_ERR_UNSUPPORTED, "stk_sdd_dsd: no kernel for this configuration");
 }

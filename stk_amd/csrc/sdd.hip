@@ -7,69 +7,9 @@
 // are staged once for four blocks.  The plan lists the tiles in the order in which the
 // workgroups take them.
 // 64-blocks run one per workgroup with the K-tile split across four wavefronts.
-#include "common.h"
-#include "gemm_core.h"
+#include "sdd_tile.h"
 
 namespace stk {
-
-struct SddArgs {
-  const elem_t* lhs;
-  int64_t lda;
-  const elem_t* rhs;
-  int64_t ldb;
-  int k;
-  elem_t* out;
-  const int32_t* offsets;  // CSR row pointers (needed for fused block rows) or null
-  const void* row_indices;
-  const void* column_indices;
-  const int32_t* block_order;
-  const int32_t* tiles;  // fusion plan: count, unused, then (first block id, rows | columns << 8) per tile; or null
-  int nnz;
-  int block_rows;
-  int idx32;
-  int activation;            // applied to the fp32 sums (an Activation value)
-  const elem_t* multiplier;  // values of a matrix with the same topology, multiplied in after the rounding; or null
-};
-
-// A tile of Cfg::A_PARTS block rows x Cfg::B_PARTS block columns.  r[i] / c[j] are the
-// block rows / columns, p[i][j] the output block ids (negative: not stored).
-template <class Cfg, int BLK, bool FULL>
-__device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem) {
-  static_assert(Cfg::PM == BLK && Cfg::PN == BLK && Cfg::A_PARTS <= 3 && Cfg::B_PARTS <= 2, "one operand part per block row / column");
-  constexpr int KT = Cfg::KT;
-  // K-major: ld is the stride between rows of the tile; MN-major: between k rows.
-  const elem_t* a0[3];
-  const elem_t* b0[2];
-#pragma unroll
-  for (int i = 0; i < 3; i++) a0[i] = g.lhs + (int64_t)r[i] * BLK * (Cfg::A_KMAJOR ? g.lda : 1);
-#pragma unroll
-  for (int j = 0; j < 2; j++) b0[j] = g.rhs + (int64_t)c[j] * BLK * (Cfg::B_KMAJOR ? g.ldb : 1);
-  const int64_t a_step = Cfg::A_KMAJOR ? KT : KT * g.lda;
-  const int64_t b_step = Cfg::B_KMAJOR ? KT : KT * g.ldb;
-  const int k = g.k;
-  const int ntiles = (k + KT - 1) / KT;
-  f32x16_t acc[Cfg::IM][Cfg::JN] = {};
-  auto tile_fn = [&](int t) {
-    const int left = k - t * KT;
-    return TilePtrs{{a0[0] + t * a_step, a0[1] + t * a_step, a0[2] + t * a_step}, {b0[0] + t * b_step, b0[1] + t * b_step}, left < KT ? left : KT};
-  };
-  if constexpr (FULL) mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem);
-  else mainloop_reg<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, BLK, BLK, smem);
-  const WaveCoords w = wave_coords<Cfg>();
-  const int m0 = wave_m0<Cfg>(w), n0 = wave_n0<Cfg>(w);
-  if constexpr (Cfg::A_PARTS == 3) {
-    // Three stored blocks below each other, one block wide; a wavefront's 96 rows may lie in two of them.
-    // Addressed as rows of the first block that run on, with the distance between the blocks added per block.
-    const int64_t at = (int64_t)p[0][0] * BLK * BLK + (int64_t)m0 * BLK + n0;
-    epilogue<Cfg, false>(acc, g.out + at, BLK, Cfg::TM - m0, BLK - n0, smem, 64, g.activation, g.multiplier ? g.multiplier + at : nullptr,
-                         m0, (int64_t)(p[1][0] - p[0][0] - 1) * BLK * BLK);
-  } else {
-    const int block = p[m0 / BLK][n0 / BLK];  // the output block this wavefront writes into
-    const int64_t at = (int64_t)(block < 0 ? 0 : block) * BLK * BLK + (int64_t)(m0 % BLK) * BLK + (n0 % BLK);
-    epilogue<Cfg, false>(acc, g.out + at, BLK, block < 0 ? 0 : BLK - (m0 % BLK), BLK - (n0 % BLK), smem, 64, g.activation,
-                         g.multiplier ? g.multiplier + at : nullptr);
-  }
-}
 
 // 128-blocks, eight wavefronts.  With a plan the workgroups take their tiles from its list: two
 // neighbouring blocks of a block row (1x2 blocks, 128x256), together with the two blocks below when
@@ -84,24 +24,7 @@ __global__ __launch_bounds__(512, 2) void sdd_fused_kernel(SddArgs g) {
     const int count = const_ints(g.tiles)[0];
     if ((int)blockIdx.x >= count) return;
     const int item = xcd_tile(blockIdx.x, count);
-    const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
-    const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
-    const bool has1 = (shape >> 8) == 2;  // an odd row ends with a tile of one block
-    const int rows = shape & 0xff, nseg = const_ints(g.offsets)[r0 + 1] - const_ints(g.offsets)[r0];
-    const int below = rows >= 2 ? p0 + nseg : -1;
-    const int c0 = uniform(load_index(g.column_indices, p0, g.idx32));
-    const int c1 = has1 ? uniform(load_index(g.column_indices, p0 + 1, g.idx32)) : c0;
-    if (rows == 3) {
-      // the last three rows of a run of identical rows: one block wide, so that the rhs panel is read once for the three
-      const int rr[3] = {r0, r0 + 1, r0 + 2}, cc[2] = {c0, c0}, pp[3][2] = {{p0, -1}, {below, -1}, {below + nseg, -1}};
-      sdd_tile<Triple, 128, FULL>(g, rr, cc, pp, smem);
-    } else if (below >= 0) {
-      const int rr[3] = {r0, r0 + 1, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {below, has1 ? below + 1 : -1}, {-1, -1}};
-      sdd_tile<Quad, 128, FULL>(g, rr, cc, pp, smem);
-    } else {
-      const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {-1, -1}, {-1, -1}};
-      sdd_tile<Pair, 128, FULL>(g, rr, cc, pp, smem);
-    }
+    sdd_plan_tile<Quad, Pair, Triple, FULL>(g, item, smem);
     return;
   }
   const int npairs = (g.nnz + 1) >> 1;
@@ -268,6 +191,53 @@ extern "C" int stk_sdd(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride
                        block_order, nnz, blocking, dtype, index_dtype, plan, STK_ACT_NONE, nullptr, stream);
 }
 
+// Checks the arguments of an sdd and turns them into the kernels' view of the problem.  STK_OK with p->empty set
+// when there is nothing to compute.
+int stk::sdd_problem(const char* who, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                     const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, int64_t m, int64_t k, int64_t n,
+                     void* out, const int32_t* offsets, const void* row_indices, const void* column_indices,
+                     const int32_t* block_order, int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                     int activation, const void* multiplier, SddProblem* p) {
+  static_assert(STK_ACT_NONE == kNoActivation && STK_ACT_RELU == kRelu && STK_ACT_GELU_TANH == kGeluTanh && STK_ACT_GELU == kGeluErf &&
+                    STK_ACT_SILU == kSilu && STK_ACT_RELU_GRAD == kReluGrad && STK_ACT_GELU_TANH_GRAD == kGeluTanhGrad &&
+                    STK_ACT_GELU_GRAD == kGeluErfGrad && STK_ACT_SILU_GRAD == kSiluGrad, "the header's activation codes are the kernels'");
+  p->empty = false;
+  if (activation < 0 || activation >= kActivations) return fail(STK_ERR_UNSUPPORTED, "%s: activation %d", who, activation);
+  if (multiplier && !aligned16(multiplier)) return fail(STK_ERR_UNSUPPORTED, "%s: multiplier needs a 16-byte aligned base", who);
+  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "%s: blocking %d (64 or 128)", who, blocking);
+  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "%s: index dtype %d", who, index_dtype);
+  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "%s: negative size", who);
+  if (m % blocking || n % blocking || k % 32)
+    return fail(STK_ERR_DIMS, "incompatible dimensions: [%lld, %lld] x [%lld, %lld] with blocking %d (m, n must be divisible by the blocking, k by 32)",
+                (long long)m, (long long)k, (long long)k, (long long)n, blocking);
+  if (k > INT32_MAX || nnz > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "%s: size exceeds 32-bit range", who);
+  if (nnz == 0) {
+    p->empty = true;
+    return STK_OK;
+  }
+  const bool ak = lhs_stride_k == 1;   // row-major lhs: K-major tile
+  const bool bk = rhs_stride_n != 1;   // .t() view of a row-major [n, k]: K-major tile
+  if (!ak && lhs_stride_m != 1) return fail(STK_ERR_UNSUPPORTED, "%s: lhs needs a unit stride", who);
+  if (bk && rhs_stride_k != 1) return fail(STK_ERR_UNSUPPORTED, "%s: rhs needs a unit stride", who);
+  const int64_t lda = ak ? lhs_stride_m : lhs_stride_k;
+  const int64_t ldb = bk ? rhs_stride_n : rhs_stride_k;
+  if (lda % 8 || ldb % 8 || !aligned16(lhs) || !aligned16(rhs) || !aligned16(out))
+    return fail(STK_ERR_UNSUPPORTED, "%s: operands need 16-byte aligned bases and leading dimensions divisible by 8", who);
+  if (lda >= (1 << 24) || ldb >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "%s: leading dimension exceeds 2^24 elements", who);
+  p->g = SddArgs{static_cast<const elem_t*>(lhs), lda, static_cast<const elem_t*>(rhs), ldb, (int)k,
+                 static_cast<elem_t*>(out), offsets, row_indices, column_indices, block_order,
+                 plan && offsets ? reinterpret_cast<const int32_t*>(plan) : nullptr, (int)nnz, (int)(m / blocking), index_dtype == STK_I32,
+                 activation, static_cast<const elem_t*>(multiplier)};
+  p->ak = ak;
+  p->bk = bk;
+  // an rhs column panel is read once per tile that holds a block of that block column: with few
+  // blocks per column (a block-diagonal MoE layout has one or two tiles per expert) it is streamed
+  // (row-major rhs only: a K-major tile uses half a cache line per K-tile and needs the line to stay)
+  p->stream_rhs = !bk && nnz <= 4 * (n / blocking);
+  return STK_OK;
+}
+
 extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
                              const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
                              int64_t m, int64_t k, int64_t n,
@@ -276,37 +246,12 @@ extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_
                              int blocking, int dtype, int index_dtype, const uint8_t* plan,
                              int activation, const void* multiplier, stk_stream_t stream) {
   using namespace stk;
-  static_assert(STK_ACT_NONE == kNoActivation && STK_ACT_RELU == kRelu && STK_ACT_GELU_TANH == kGeluTanh && STK_ACT_GELU == kGeluErf &&
-                    STK_ACT_SILU == kSilu && STK_ACT_RELU_GRAD == kReluGrad && STK_ACT_GELU_TANH_GRAD == kGeluTanhGrad &&
-                    STK_ACT_GELU_GRAD == kGeluErfGrad && STK_ACT_SILU_GRAD == kSiluGrad, "the header's activation codes are the kernels'");
-  if (activation < 0 || activation >= kActivations) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: activation %d", activation);
-  if (multiplier && !aligned16(multiplier)) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: multiplier needs a 16-byte aligned base");
-  if (blocking != 64 && blocking != 128) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: blocking %d (64 or 128)", blocking);
-  if (dtype != STK_F16 && dtype != STK_BF16) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: dtype %d", dtype);
-  if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: index dtype %d", index_dtype);
-  if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "stk_sdd: negative size");
-  if (m % blocking || n % blocking || k % 32)
-    return fail(STK_ERR_DIMS, "incompatible dimensions: [%lld, %lld] x [%lld, %lld] with blocking %d (m, n must be divisible by the blocking, k by 32)",
-                (long long)m, (long long)k, (long long)k, (long long)n, blocking);
-  if (k > INT32_MAX || nnz > INT32_MAX) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: size exceeds 32-bit range");
-  if (nnz == 0) return STK_OK;
-  const bool ak = lhs_stride_k == 1;   // row-major lhs: K-major tile
-  const bool bk = rhs_stride_n != 1;   // .t() view of a row-major [n, k]: K-major tile
-  if (!ak && lhs_stride_m != 1) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: lhs needs a unit stride");
-  if (bk && rhs_stride_k != 1) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: rhs needs a unit stride");
-  const int64_t lda = ak ? lhs_stride_m : lhs_stride_k;
-  const int64_t ldb = bk ? rhs_stride_n : rhs_stride_k;
-  if (lda % 8 || ldb % 8 || !aligned16(lhs) || !aligned16(rhs) || !aligned16(out))
-    return fail(STK_ERR_UNSUPPORTED, "stk_sdd: operands need 16-byte aligned bases and leading dimensions divisible by 8");
-  if (lda >= (1 << 24) || ldb >= (1 << 24)) return fail(STK_ERR_UNSUPPORTED, "stk_sdd: leading dimension exceeds 2^24 elements");
-  const SddArgs g{static_cast<const elem_t*>(lhs), lda, static_cast<const elem_t*>(rhs), ldb, (int)k,
-                  static_cast<elem_t*>(out), offsets, row_indices, column_indices, block_order,
-                  plan && offsets ? reinterpret_cast<const int32_t*>(plan) : nullptr, (int)nnz, (int)(m / blocking), index_dtype == STK_I32,
-                  activation, static_cast<const elem_t*>(multiplier)};
-  // an rhs column panel is read once per tile that holds a block of that block column: with few
-  // blocks per column (a block-diagonal MoE layout has one or two tiles per expert) it is streamed
-  // (row-major rhs only: a K-major tile uses half a cache line per K-tile and needs the line to stay)
-  const bool stream_rhs = !bk && nnz <= 4 * (n / blocking);
+  SddProblem problem;
+  const int rc = sdd_problem("stk_sdd", lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, offsets, row_indices,
+                             column_indices, block_order, nnz, blocking, dtype, index_dtype, plan, activation, multiplier, &problem);
+  if (rc != STK_OK || problem.empty) return rc;
+  const SddArgs& g = problem.g;
+  const bool ak = problem.ak, bk = problem.bk, stream_rhs = problem.stream_rhs;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define STK_SDD_CASE(BF, BLK, AK, BK)                                         \
   if ((dtype == STK_BF16) == BF && blocking == BLK && ak == AK && bk == BK) { \

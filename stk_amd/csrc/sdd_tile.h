@@ -1,0 +1,104 @@
+// Tile functions of stk_sdd, shared by its kernels (sdd.hip) and by the launch that computes an sdd and a dsd on
+// the same topology together (grad.hip).
+#pragma once
+#include "common.h"
+#include "gemm_core.h"
+
+namespace stk {
+
+struct SddArgs {
+  const elem_t* lhs;
+  int64_t lda;
+  const elem_t* rhs;
+  int64_t ldb;
+  int k;
+  elem_t* out;
+  const int32_t* offsets;  // CSR row pointers (needed for fused block rows) or null
+  const void* row_indices;
+  const void* column_indices;
+  const int32_t* block_order;
+  const int32_t* tiles;  // fusion plan: count, unused, then (first block id, rows | columns << 8) per tile; or null
+  int nnz;
+  int block_rows;
+  int idx32;
+  int activation;            // applied to the fp32 sums (an Activation value)
+  const elem_t* multiplier;  // values of a matrix with the same topology, multiplied in after the rounding; or null
+};
+
+// A tile of Cfg::A_PARTS block rows x Cfg::B_PARTS block columns.  r[i] / c[j] are the
+// block rows / columns, p[i][j] the output block ids (negative: not stored).
+template <class Cfg, int BLK, bool FULL>
+__device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem) {
+  static_assert(Cfg::PM == BLK && Cfg::PN == BLK && Cfg::A_PARTS <= 3 && Cfg::B_PARTS <= 2, "one operand part per block row / column");
+  constexpr int KT = Cfg::KT;
+  // K-major: ld is the stride between rows of the tile; MN-major: between k rows.
+  const elem_t* a0[3];
+  const elem_t* b0[2];
+#pragma unroll
+  for (int i = 0; i < 3; i++) a0[i] = g.lhs + (int64_t)r[i] * BLK * (Cfg::A_KMAJOR ? g.lda : 1);
+#pragma unroll
+  for (int j = 0; j < 2; j++) b0[j] = g.rhs + (int64_t)c[j] * BLK * (Cfg::B_KMAJOR ? g.ldb : 1);
+  const int64_t a_step = Cfg::A_KMAJOR ? KT : KT * g.lda;
+  const int64_t b_step = Cfg::B_KMAJOR ? KT : KT * g.ldb;
+  const int k = g.k;
+  const int ntiles = (k + KT - 1) / KT;
+  f32x16_t acc[Cfg::IM][Cfg::JN] = {};
+  auto tile_fn = [&](int t) {
+    const int left = k - t * KT;
+    return TilePtrs{{a0[0] + t * a_step, a0[1] + t * a_step, a0[2] + t * a_step}, {b0[0] + t * b_step, b0[1] + t * b_step}, left < KT ? left : KT};
+  };
+  if constexpr (FULL) mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem);
+  else mainloop_reg<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, BLK, BLK, smem);
+  const WaveCoords w = wave_coords<Cfg>();
+  const int m0 = wave_m0<Cfg>(w), n0 = wave_n0<Cfg>(w);
+  if constexpr (Cfg::A_PARTS == 3) {
+    // Three stored blocks below each other, one block wide; a wavefront's 96 rows may lie in two of them.
+    // Addressed as rows of the first block that run on, with the distance between the blocks added per block.
+    const int64_t at = (int64_t)p[0][0] * BLK * BLK + (int64_t)m0 * BLK + n0;
+    epilogue<Cfg, false>(acc, g.out + at, BLK, Cfg::TM - m0, BLK - n0, smem, 64, g.activation, g.multiplier ? g.multiplier + at : nullptr,
+                         m0, (int64_t)(p[1][0] - p[0][0] - 1) * BLK * BLK);
+  } else {
+    const int block = p[m0 / BLK][n0 / BLK];  // the output block this wavefront writes into
+    const int64_t at = (int64_t)(block < 0 ? 0 : block) * BLK * BLK + (int64_t)(m0 % BLK) * BLK + (n0 % BLK);
+    epilogue<Cfg, false>(acc, g.out + at, BLK, block < 0 ? 0 : BLK - (m0 % BLK), BLK - (n0 % BLK), smem, 64, g.activation,
+                         g.multiplier ? g.multiplier + at : nullptr);
+  }
+}
+
+// The tile `item` of the plan's list (128-blocks): two neighbouring blocks of a block row (1x2 blocks, 128x256),
+// together with the two blocks below when the next row repeats this one (2x2 blocks, 256x256), or one block with
+// the two below it for the last three rows of a run of odd length (3x1 blocks, 384x128).
+template <class Quad, class Pair, class Triple, bool FULL>
+__device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* smem) {
+  const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
+  const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
+  const bool has1 = (shape >> 8) == 2;  // an odd row ends with a tile of one block
+  const int rows = shape & 0xff, nseg = const_ints(g.offsets)[r0 + 1] - const_ints(g.offsets)[r0];
+  const int below = rows >= 2 ? p0 + nseg : -1;
+  const int c0 = uniform(load_index(g.column_indices, p0, g.idx32));
+  const int c1 = has1 ? uniform(load_index(g.column_indices, p0 + 1, g.idx32)) : c0;
+  if (rows == 3) {
+    // the last three rows of a run of identical rows: one block wide, so that the rhs panel is read once for the three
+    const int rr[3] = {r0, r0 + 1, r0 + 2}, cc[2] = {c0, c0}, pp[3][2] = {{p0, -1}, {below, -1}, {below + nseg, -1}};
+    sdd_tile<Triple, 128, FULL>(g, rr, cc, pp, smem);
+  } else if (below >= 0) {
+    const int rr[3] = {r0, r0 + 1, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {below, has1 ? below + 1 : -1}, {-1, -1}};
+    sdd_tile<Quad, 128, FULL>(g, rr, cc, pp, smem);
+  } else {
+    const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {-1, -1}, {-1, -1}};
+    sdd_tile<Pair, 128, FULL>(g, rr, cc, pp, smem);
+  }
+}
+
+// A checked sdd: the kernels' arguments and the operands' layouts.
+struct SddProblem {
+  SddArgs g;
+  bool ak, bk, stream_rhs, empty;
+};
+int sdd_problem(const char* who, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, int64_t m, int64_t k, int64_t n,
+                void* out, const int32_t* offsets, const void* row_indices, const void* column_indices,
+                const int32_t* block_order, int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                int activation, const void* multiplier, SddProblem* p);
+
+}  // namespace stk

@@ -500,15 +500,22 @@ def test_results_do_not_depend_on_the_fusion_plan(monkeypatch, b):
     U.assert_close(plain[1], O.dsd(topo.shape, U.np32(h0.data), topo, False, U.np32(w2)), dtype, "dsd without plan")
 
 
-@pytest.mark.parametrize("dtype,blocking,hidden", [(torch.bfloat16, 128, 1024), (torch.float16, 128, 512), (torch.bfloat16, 128, 256),
-                                                   (torch.float16, 64, 1024)])
-def test_both_gradients_of_sdd_in_one_call(dtype, blocking, hidden, monkeypatch):
+_JOINT_TOKENS = [300, 0, 129, 384, 640, 128, 77, 256, 512, 1000, 40, 896]
+# (dtype, blocking, hidden, ffn, tokens per expert); the first two have the work per compute unit that the joint launches
+# ask for (nonzero blocks x hidden / 128 >= 40 x 256 compute units), the others run the two products one after the other
+_JOINT_CASES = [(torch.bfloat16, 128, 1024, 4096, _JOINT_TOKENS + [512, 384, 640, 512]),
+                (torch.float16, 128, 1024, 4096, _JOINT_TOKENS + [256] * 8),
+                (torch.float16, 128, 512, 2048, _JOINT_TOKENS), (torch.bfloat16, 128, 256, 2048, _JOINT_TOKENS),
+                (torch.bfloat16, 128, 384, 4096, _JOINT_TOKENS + [512] * 6), (torch.float16, 64, 1024, 2048, _JOINT_TOKENS)]
+
+
+@pytest.mark.parametrize("dtype,blocking,hidden,ffn,tokens", _JOINT_CASES)
+def test_both_gradients_of_sdd_in_one_call(dtype, blocking, hidden, ffn, tokens, monkeypatch):
     # stk_dsd_dds: dS rhs^T and lhs^T dS from one call (one launch for 128-blocks with enough work; otherwise the two
     # products one after the other) against the oracle's dsd and dds, and bit for bit against the separate launches
     from stk_amd.backend import autograd, hip_kernels
     monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
-    tokens = np.array([300, 0, 129, 384, 640, 128, 77, 256, 512, 1000, 40, 896])
-    topo, tm, x, w1, w2 = _dmoe_case(tokens, hidden, 2048, blocking, dtype, 31)
+    topo, tm, x, w1, w2 = _dmoe_case(np.array(tokens), hidden, ffn, blocking, dtype, 31)
     g = torch.Generator().manual_seed(32)
     ds = (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV)
     dsm = stk.Matrix(tm.size(), ds, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
@@ -529,6 +536,44 @@ def test_both_gradients_of_sdd_in_one_call(dtype, blocking, hidden, monkeypatch)
         grads[joint] = (xs.grad, ws.grad)
     assert torch.equal(grads[True][0], grads[False][0]) and torch.equal(grads[True][1], grads[False][1])
     assert torch.equal(grads[True][0], dx) and torch.equal(grads[True][1], dw1)
+
+
+@pytest.mark.parametrize("transpose_a", [False, True])
+@pytest.mark.parametrize("dtype,blocking,hidden,ffn,tokens", _JOINT_CASES)
+def test_both_gradients_of_dsd_in_one_call(dtype, blocking, hidden, ffn, tokens, transpose_a, monkeypatch):
+    # stk_sdd_dsd: dy rhs^T on the pattern and op(S)^T dy from one call (one launch for 128-blocks with enough work;
+    # otherwise the two products one after the other) against the oracle's sdd and dsd, and bit for bit against the
+    # separate launches
+    from stk_amd.backend import autograd, hip_kernels
+    monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
+    topo, tm, x, w1, w2 = _dmoe_case(np.array(tokens), hidden, ffn, blocking, dtype, 33)
+    g = torch.Generator().manual_seed(34)
+    s = (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV)
+    sm = stk.Matrix(tm.size(), s, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
+    rows, cols = tm.size()
+    meta = (tm.offsets, tm.row_indices, tm.column_indices, tm.offsets_t, tm.column_indices_t, tm.block_offsets_t)
+    # y = S w2 [rows, hidden] or y = S^T x [cols, hidden]
+    rhs = x if transpose_a else w2
+    dy = (torch.randn(cols if transpose_a else rows, hidden, generator=g) * 0.05).to(dtype).to(DEV)
+    ds = torch.full(tuple(s.shape), float("nan"), dtype=dtype, device=DEV)
+    drhs = torch.full(tuple(rhs.shape), float("nan"), dtype=dtype, device=DEV)
+    lhs, rhs_sdd = (rhs, dy.t()) if transpose_a else (dy, rhs.t())
+    hip_kernels.sdd_dsd(tm.size(), lhs, rhs_sdd, ds, s, *meta, not transpose_a, dy, drhs)
+    U.assert_close(ds, O.sdd(U.np32(lhs), U.np32(rhs_sdd), topo), dtype, "dy rhs^T on the pattern")
+    logical = topo.shape if transpose_a else (cols, rows)
+    U.assert_close(drhs, O.dsd(logical, U.np32(s), topo, not transpose_a, U.np32(dy)), dtype, "op(S)^T dy")
+    assert torch.equal(ds, stk.ops.sdd(lhs, rhs_sdd, tm).data)
+    assert torch.equal(drhs, stk.ops.dsd(sm if transpose_a else sm.t(), dy))
+    # through autograd: the gradients of dsd with the joint call and with two launches
+    grads = {}
+    for joint in (True, False):
+        monkeypatch.setattr(autograd, "JOINT_GRADIENTS", joint)
+        ss, rs = s.detach().clone().requires_grad_(True), rhs.detach().clone().requires_grad_(True)
+        m = stk.Matrix(tm.size(), ss, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
+        stk.ops.dsd(m.t() if transpose_a else m, rs).backward(dy)
+        grads[joint] = (ss.grad, rs.grad)
+    assert torch.equal(grads[True][0], grads[False][0]) and torch.equal(grads[True][1], grads[False][1])
+    assert torch.equal(grads[True][0], ds) and torch.equal(grads[True][1], drhs)
 
 
 def test_gradients_side_by_side_equal_gradients_one_after_the_other(monkeypatch):
