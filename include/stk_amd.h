@@ -75,6 +75,15 @@ const char* stk_last_error(void);
 int stk_abi_version(void);
 
 /*
+ * *id = identifier of the graph capture under way on `stream`, 0 when the stream is not capturing.  No counterpart
+ * in the reference (its launches go through Triton, which knows nothing of captures): it is for bindings that cache
+ * device buffers between calls, as the Python boundary does with fusion plans and the dsd workspace.  A buffer that
+ * is allocated or filled while a capture is under way exists only in that graph's replays, so such a cache must not
+ * hand it to launches outside that capture.
+ */
+int stk_stream_capture_id(stk_stream_t stream, uint64_t* id);
+
+/*
  * Fusion plan of a topology: which neighbouring block rows (and block columns) repeat
  * each other's pattern, so that two of them (for stk_dsd also the last three of an odd
  * run) can be computed together as one tile and share every read of the other operand.

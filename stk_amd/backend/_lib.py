@@ -22,6 +22,7 @@ _p, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_si
 SIGNATURES = {
     "stk_last_error": (ctypes.c_char_p, []),
     "stk_abi_version": (_int, []),
+    "stk_stream_capture_id": (_int, [_p, _p]),
     "stk_plan_bytes": (_sz, [_i64, _i64, _i64]),
     "stk_build_plan": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _int, _int, _p, _sz, _p]),
     "stk_sdd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _p]),

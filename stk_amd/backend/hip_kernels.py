@@ -11,6 +11,7 @@ Everything here needs tensors on a ROCm device and launches on torch's current
 stream without synchronising (to_sparse reads one int back, as the reference's
 torch.nonzero does).  Nothing falls back to another implementation.
 """
+import ctypes
 import threading
 
 import torch
@@ -32,6 +33,15 @@ def _stream(device=None):
     if _raw_stream is not None and _raw_device is not None:
         return _raw_stream(_raw_device() if device is None or device.index is None else device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def _capture_id(device=None):
+    """Identifier of the graph capture under way on the current stream of `device`, 0 outside captures.  A buffer
+    allocated or filled while a capture is under way exists only in that graph's replays: the caches below keep
+    such a buffer apart from launches outside that capture."""
+    out = ctypes.c_uint64(0)
+    _lib.check(_lib.load().stk_stream_capture_id(_stream(device), ctypes.byref(out)))
+    return out.value
 
 
 class _on_device:
@@ -128,14 +138,15 @@ def _plan_cache_get(tensors, blocking):
     return cached
 
 
-def _plan_cache_put(tensors, blocking, plan, stream_handle, built):
+def _plan_cache_put(tensors, blocking, plan, stream_handle, built, capture):
     """Remembers `plan` on tensors[0]; tensors without a version counter (made under inference mode)
-    cannot be watched for in-place changes and are not cached."""
+    cannot be watched for in-place changes and are not cached.  `capture`: the graph capture the plan was built in
+    (0: none)."""
     versions = tuple(_version_of(t) for t in tensors)
     if None in versions:
         return False
     try:
-        tensors[0]._stk_plan = (tuple(tensors[1:]), plan, blocking, stream_handle, built, versions)
+        tensors[0]._stk_plan = (tuple(tensors[1:]), plan, blocking, stream_handle, built, versions, capture)
     except AttributeError:
         return False
     return True
@@ -146,16 +157,28 @@ def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, 
     transpose metadata is given, of the block columns): which neighbouring lines
     repeat each other and are computed as one 256-wide tile.  Depends on the
     topology only, so it is cached on the `offsets` tensor and rebuilt when one of
-    the index tensors has been replaced or modified in place."""
+    the index tensors has been replaced or modified in place.
+
+    Under a graph capture: a plan built before the capture is used as it is (on another stream than the one that
+    built it without waiting for the build, which a capture cannot do: the build must be complete when the capture
+    starts, as it is after the synchronisation with which torch.cuda.graph() begins); a plan built inside a capture
+    serves that capture only, and launches outside it build their own."""
     _need_gpu(offsets, column_indices)
     want_cols = offsets_t is not None and column_indices_t is not None
     tensors = (offsets, column_indices) + ((offsets_t, column_indices_t) if want_cols else ())
     cached = _plan_cache_get(tensors, blocking)
     if cached is not None:
-        if cached[3] != _stream(offsets.device):
-            # built on another stream: what this one launches next comes after the build
-            torch.cuda.current_stream(offsets.device).wait_event(cached[4])
-        return cached[1]
+        handle, built_in = _stream(offsets.device), cached[6]
+        if built_in == 0 and cached[3] == handle:
+            return cached[1]
+        capture = _capture_id(offsets.device)
+        if built_in in (0, capture):
+            if cached[3] != handle and (built_in != 0 or capture == 0):
+                # built on another stream: what this one launches next comes after the build
+                torch.cuda.current_stream(offsets.device).wait_event(cached[4])
+            return cached[1]
+    else:
+        capture = _capture_id(offsets.device)
     block_rows = offsets.numel() - 1
     block_cols = offsets_t.numel() - 1 if want_cols else 0
     lib = _lib.load()
@@ -172,7 +195,7 @@ def fusion_plan(offsets, column_indices, offsets_t=None, column_indices_t=None, 
     stream = torch.cuda.current_stream(offsets.device)
     built = torch.cuda.Event()
     built.record(stream)
-    _plan_cache_put(tensors, blocking, plan, stream.cuda_stream, built)
+    _plan_cache_put(tensors, blocking, plan, stream.cuda_stream, built, capture)
     return plan
 
 
@@ -272,10 +295,14 @@ def _dsd_workspace(device, m, n, blocking):
     counters = lib.stk_dsd_workspace_counter_bytes()
     nbytes = counters + DSD_WORKSPACE_SLOTS * lib.stk_dsd_workspace_slot_bytes()
     if entry is None or entry[0].numel() != nbytes:
+        if _capture_id(device):
+            return None     # a buffer made inside a capture would belong to that graph: this launch runs uncut
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
         ws[:counters].zero_()   # the slots behind the counters need no initial value
         entry = _dsd_workspaces[key] = [ws, torch.cuda.current_stream(device)]
-    elif entry[1].cuda_stream != handle:
+    elif entry[1].cuda_stream != handle and not _capture_id(device):
+        # (a capture cannot wait for work outside it: replays of a graph with such a launch must not overlap other
+        # dsd launches of the device, which holds when they are issued to the stream those use)
         stream = torch.cuda.current_stream(device)
         stream.wait_stream(entry[1])   # launches that share a workspace must not overlap
         entry[1] = stream
@@ -485,6 +512,9 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
     offsets, mask = scratch[:4 * (br + 1)].view(torch.int32), scratch[4 * (br + 1):]
     lib = _lib.load()
     with _on_device(dev):
+        if _capture_id(dev):
+            raise RuntimeError("to_sparse sizes its result by the number of nonzero blocks, which the host reads back: "
+                               "it cannot be captured into a graph")
         # nnz arrives in pinned host memory, written by the counting kernel: one wait, no copy to launch
         buffers = _nnz_buffers.__dict__.setdefault("of_device", {})
         nnz_host = buffers.get(dev.index)

@@ -508,6 +508,20 @@ using namespace stk;
 extern "C" const char* stk_last_error(void) { return error_buffer(); }
 extern "C" int stk_abi_version(void) { return STK_AMD_ABI_VERSION; }
 
+extern "C" int stk_stream_capture_id(stk_stream_t stream, uint64_t* id) {
+  if (!id) return fail(STK_ERR_DIMS, "stk_stream_capture_id: null output");
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long capture = 0;
+  *id = 0;
+  const hipError_t e = hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &capture);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // the query's own failure is not left behind for the next launch check
+    return fail(STK_ERR_HIP, "stk_stream_capture_id: %s", hipGetErrorString(e));
+  }
+  if (status == hipStreamCaptureStatusActive) *id = capture ? (uint64_t)capture : UINT64_MAX;
+  return STK_OK;
+}
+
 extern "C" int stk_row_indices(const int32_t* offsets, int64_t block_rows, int64_t nnz, void* out, int index_dtype,
                                stk_stream_t stream) {
   if (index_dtype != STK_I16 && index_dtype != STK_I32) return fail(STK_ERR_UNSUPPORTED, "stk_row_indices: index dtype %d", index_dtype);

@@ -207,7 +207,7 @@ def test_fusion_plan_cache_is_tied_to_the_index_tensors_it_was_built_from():
     ot, cit = torch.arange(0, 20, 4, dtype=torch.int32), torch.tensor([0, 1, 2, 3] * 4, dtype=torch.int16)
     plan = object()
     assert hk._plan_cache_get((offsets, ci), 128) is None
-    assert hk._plan_cache_put((offsets, ci, ot, cit), 128, plan, 7, None)
+    assert hk._plan_cache_put((offsets, ci, ot, cit), 128, plan, 7, None, 0)
     assert hk._plan_cache_get((offsets, ci, ot, cit), 128)[1] is plan
     assert hk._plan_cache_get((offsets, ci), 128)[1] is plan               # a request without the transpose metadata
     assert hk._plan_cache_get((offsets, ci, ot, cit), 64) is None          # another blocking
@@ -224,11 +224,11 @@ def test_fusion_plan_cache_is_tied_to_the_index_tensors_it_was_built_from():
     held[0] = 5
     assert hk._plan_cache_get((offsets, held, ot, cit), 128) is None
     # a plan built without the transpose metadata does not serve a request with it
-    assert hk._plan_cache_put((offsets, held), 128, plan, 7, None)
+    assert hk._plan_cache_put((offsets, held), 128, plan, 7, None, 0)
     assert hk._plan_cache_get((offsets, held, ot, cit), 128) is None
     # tensors made under inference mode keep no version counter: never cached, and asking does not raise
     with torch.inference_mode():
         frozen = torch.arange(0, 20, 4, dtype=torch.int32)
         fci = torch.zeros(16, dtype=torch.int16)
-    assert not hk._plan_cache_put((frozen, fci), 128, plan, 7, None)
+    assert not hk._plan_cache_put((frozen, fci), 128, plan, 7, None, 0)
     assert hk._plan_cache_get((frozen, fci), 128) is None
