@@ -141,3 +141,59 @@ def test_a_plan_built_inside_a_capture_serves_that_capture_only(monkeypatch):
     with pytest.raises(RuntimeError, match="cannot be captured"):
         with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
             stk.ops.to_sparse(y, 128)
+
+
+def test_a_routed_layer_replays_from_a_graph_with_new_expert_choices():
+    # route -> gather -> topology -> sdd -> dsd -> weighted scatter and its backward pass in one graph: with the rows of the
+    # padded layout fixed at their upper bound nothing is read back to the host, and the topology, its transpose
+    # metadata and its fusion plan are rebuilt by every replay from the expert choices of that replay
+    tokens, experts, blocking, hidden, ffn, top_k = 4096, 16, 128, 1024, 4096, 2
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(47)
+    capacity = stk.ops.route_capacity(tokens * top_k, experts, blocking)
+    top = torch.zeros(tokens, top_k, dtype=torch.int32, device=DEV)
+    x = _fresh(torch.empty(tokens, hidden, dtype=dtype, device=DEV), g, 0.5).requires_grad_(True)
+    w1 = _fresh(torch.empty(hidden, experts * ffn, dtype=dtype, device=DEV), g, 0.05).requires_grad_(True)
+    w2 = _fresh(torch.empty(experts * ffn, hidden, dtype=dtype, device=DEV), g, 0.05).requires_grad_(True)
+    weights = torch.rand(tokens, top_k, generator=g).to(DEV).requires_grad_(True)
+    grad = _fresh(torch.empty(tokens, hidden, dtype=dtype, device=DEV), g, 1.0)
+    leaves = (x, w1, w2, weights)
+
+    def layer(padded_rows):
+        r = stk.ops.route(top, experts, blocking, padded_rows)
+        padded = stk.ops.padded_gather(x, r)
+        topo = stk.ops.dmoe_topology(r.padded_bins, blocking, padded.shape[0] // blocking, ffn // blocking, dtype=dtype)
+        return stk.ops.padded_scatter(stk.ops.dsd(stk.ops.sdd(padded, w1, topo), w2), r, weights)
+
+    def choices(seed, skew):
+        p = torch.arange(1, experts + 1, dtype=torch.float64).pow(-skew)
+        picks = torch.multinomial(p.expand(tokens, experts), top_k, generator=torch.Generator().manual_seed(seed))
+        return picks.to(torch.int32).to(DEV)
+
+    top.copy_(choices(1, 0.0))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            layer(capacity).backward(grad)
+            for t in leaves:
+                t.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out = layer(capacity)
+        out.backward(grad)
+    grads = [t.grad for t in leaves]
+    for replay, skew in enumerate((0.0, 1.2, 3.0)):
+        top.copy_(choices(10 + replay, skew))      # uniform, skewed, and nearly everything on two experts
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [out.clone()] + [t.clone() for t in grads]
+        eager = layer(capacity)
+        want = [eager] + list(torch.autograd.grad(eager, leaves, grad))
+        exact = layer(None)                        # rows read back from the device: no surplus rows behind the last expert
+        torch.cuda.synchronize()
+        for p, q, what in zip(got, want, ("out", "dx", "dW1", "dW2", "dweights")):
+            assert torch.equal(p, q), (what, replay)
+        U.assert_close(got[0], U.np32(exact), dtype, "surplus rows change nothing")
+        assert got[0].float().abs().sum() > 0
