@@ -295,6 +295,36 @@ def gradient_pair_times(topo, x, w1, calls):
     return out
 
 
+def dsd_gradient_pair_times(topo, x, w1, w2, calls):
+    """The two gradients of dsd(h, W2) on the benchmark topology, sdd(dy, W2^T) on the pattern and dsd(h^T, dy), as the one
+    launch of stk_sdd_dsd and as two launches (stk_sdd, stk_dsd without its workspace); `calls` times each, back to back."""
+    from stk_amd.backend import hip_kernels
+    import stk_amd as stk
+    h = stk.ops.sdd(x, w1, topo).data
+    dy = torch.empty_like(x).normal_(0, 0.02)
+    meta = (topo.offsets, topo.row_indices, topo.column_indices, topo.offsets_t, topo.column_indices_t, topo.block_offsets_t)
+    dh, dw2 = torch.empty_like(h), torch.empty_like(w2)
+    rows, cols = topo.size()
+    slicing, hip_kernels.SLICE_LAST_ROUND = hip_kernels.SLICE_LAST_ROUND, False
+
+    def joint():
+        hip_kernels.sdd_dsd((rows, cols), dy, w2.t(), dh, h, *meta, True, dy, dw2)
+
+    def two():
+        hip_kernels.sdd(dy, w2.t(), (rows, cols), dh, topo.offsets, topo.row_indices, topo.column_indices, block_order=topo.block_offsets_t)
+        hip_kernels.dsd((cols, rows), h, *meta, True, dy, dw2)
+
+    try:
+        for fn in (joint, two):
+            for _ in range(3):
+                fn()
+        out = {"joint_launch_ms": time_batch(joint, calls), "two_launches_ms": time_batch(two, calls)}
+    finally:
+        hip_kernels.SLICE_LAST_ROUND = slicing
+    out["note"] = "sdd(dy,W2^T) + dsd(h^T,dy): stk_sdd_dsd against stk_sdd followed by stk_dsd (no workspace), back to back"
+    return out
+
+
 def _expert_choices(name, seed=0):
     """[tokens, top_k] int32 expert choices of the dMoE configurations of BASELINE.json."""
     g = torch.Generator().manual_seed(seed)
@@ -427,7 +457,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB -> 1 GiB elementwise kernel (torch.neg), the known-size reference for the HBM counters")
     ap.add_argument("--gradient-pair-only", action="store_true",
-                    help="run only the two operand gradients of sdd, as one launch and as two (for the counter profiles)")
+                    help="run only the gradient pairs of sdd and of dsd, each as one launch and as two (for the counter profiles)")
     ap.add_argument("--configs", default="2,4,5,5skew",
                     help="comma-separated other configurations of BASELINE.json to time as well (2, 4, 5, 5skew); 'none' leaves them out")
     args = ap.parse_args()
@@ -453,7 +483,8 @@ def main():
 
     if args.gradient_pair_only:
         with torch.no_grad():
-            print(json.dumps({"sdd_gradient_pair": gradient_pair_times(topo, x, w1, max(args.steps, 1))}))
+            print(json.dumps({"sdd_gradient_pair": gradient_pair_times(topo, x, w1, max(args.steps, 1)),
+                              "dsd_gradient_pair": dsd_gradient_pair_times(topo, x, w1, w2, max(args.steps, 1))}))
         return
 
     names = ("sdd", "dsd", "dds")
@@ -534,6 +565,10 @@ def main():
             gradient_pair = gradient_pair_times(topo, x, w1, args.steps)
         except Exception as exc:  # noqa: BLE001
             gradient_pair = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+        try:
+            dsd_gradient_pair = dsd_gradient_pair_times(topo, x, w1, w2, args.steps)
+        except Exception as exc:  # noqa: BLE001
+            dsd_gradient_pair = {"error": f"{type(exc).__name__}: {exc}"[:300]}
         gc.enable()
 
         others = {}
@@ -593,6 +628,7 @@ def main():
         "roofline": roof,
         "routing": routing,
         "sdd_gradient_pair": gradient_pair,
+        "dsd_gradient_pair": dsd_gradient_pair,
     }
     if others:
         result["other_configs"] = others
