@@ -117,8 +117,10 @@ extern "C" int stk_dsd_dds(int64_t m, int64_t k,
   rc = dds_problem("stk_dsd_dds", m_dds, m, k, lhs, lhs_stride_m, lhs_stride_k, data, offsets, column_indices, offsets_t, column_indices_t,
                    block_offsets_t, 0, out_dds, out_dds_stride, nnz, blocking, dtype, index_dtype, plan, &dds);
   if (rc != STK_OK) return rc;
+  // (the grid of the one launch - an upper bound on the tiles of both products - must be a 32-bit count)
   const bool together = plan && blocking == 128 && nnz > 0 && !dsd.empty && !dds.empty && dsd.bk && !dds.ak && n_dsd % 256 == 0 &&
-                        m_dds % 256 == 0 && !dsd.g.small && !dds.g.small;
+                        m_dds % 256 == 0 && !dsd.g.small && !dds.g.small &&
+                        (int64_t)dsd.g.block_rows * (n_dsd / 256) + (int64_t)dds.g.block_cols * (m_dds / 256) <= INT32_MAX;
   if (!together) {
     // shapes or layouts the joint launch has no tiles for: the two products one after the other
     rc = stk_dsd(m, k, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k, rhs_stride_n,
@@ -158,7 +160,8 @@ extern "C" int stk_sdd_dsd(int64_t m, int64_t n,
                    rhs_dsd, rhs_dsd_stride_k, rhs_dsd_stride_n, out_dsd, out_dsd_stride, nnz, blocking, dtype, index_dtype, plan, &dsd);
   if (rc != STK_OK) return rc;
   const bool together = plan && blocking == 128 && !sdd.empty && !dsd.empty && sdd.g.tiles && nnz > compute_units() && sdd.ak && sdd.bk &&
-                        k_sdd % 64 == 0 && !dsd.bk && n_dsd % 256 == 0 && !dsd.g.small;
+                        k_sdd % 64 == 0 && !dsd.bk && n_dsd % 256 == 0 && !dsd.g.small &&
+                        sdd_max_tiles(sdd.g.block_rows, nnz) + (int64_t)dsd.g.block_rows * (n_dsd / 256) <= INT32_MAX;
   if (!together) {
     // shapes or layouts the joint launch has no tiles for: the two products one after the other
     rc = stk_sdd(lhs, lhs_stride_m, lhs_stride_k, rhs_sdd, rhs_sdd_stride_k, rhs_sdd_stride_n, m, k_sdd, n, out_sdd, offsets, row_indices,
