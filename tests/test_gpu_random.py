@@ -1,0 +1,121 @@
+"""Random differential test: the three products and all their gradients on random topologies against the dense
+fp32 comparator that the tolerance is stated for (to_dense + torch.matmul, masked to the topology), on the GPU.
+
+Each case draws a block size, a value type, an index type, a pattern (uniformly random blocks, runs of identical
+rows, block-diagonal experts with and without empty experts), transposes for both operands and the dense extents.
+The seeds are fixed, so a failure names a case that can be run again.  Tolerance: |got - want| <= atol + 1e-2 |want|
+with atol 1e-2 (bfloat16) / 5e-3 (float16), and, because operands of this size leave that bound loose, also
+max |got - want| <= 2^-6 (2^-9) of the largest |want| - a dropped or doubled block fails it.
+"""
+import numpy as np
+import pytest
+import torch
+
+import stk_amd as stk
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+CASES_PER_TEST = 40
+
+
+def _check(name, got, want, dtype, info):
+    got, want = got.float(), want.float()
+    atol = 1e-2 if dtype == torch.bfloat16 else 5e-3
+    err = (got - want).abs()
+    assert torch.isfinite(got).all(), (name, info)
+    assert bool((err <= atol + 1e-2 * want.abs()).all()), (name, info, err.max().item())
+    scale_free = 2.0 ** -6 if dtype == torch.bfloat16 else 2.0 ** -9
+    assert err.max().item() <= scale_free * want.abs().max().item() + 1e-30, (name, info, err.max().item(), want.abs().max().item())
+
+
+def _pattern(rng):
+    kind = rng.choice(["random", "runs", "experts", "wide experts"])
+    if kind == "random":
+        mask = rng.rand(int(rng.randint(1, 24)), int(rng.randint(1, 24))) < rng.choice([0.1, 0.3, 0.6, 1.0])
+    elif kind == "runs":      # runs of identical block rows (fused tiles), some of them empty
+        rows, cols = int(rng.randint(2, 40)), int(rng.randint(2, 24))
+        patterns = rng.rand(4, cols) < 0.5
+        mask = patterns[np.sort(rng.randint(0, 4, rows))]
+    else:                     # block-diagonal: experts of 0 .. 8 block rows
+        experts = int(rng.randint(1, 12))
+        per = int(rng.choice([1, 2, 4, 8] if kind == "experts" else [16, 32]))
+        rows_of = rng.randint(0, 5 if kind == "experts" else 9, experts)
+        if rows_of.sum() == 0:
+            rows_of[0] = 1
+        mask = np.zeros((int(rows_of.sum()), experts * per), bool)
+        r0 = 0
+        for e, n in enumerate(rows_of):
+            mask[r0:r0 + n, e * per:(e + 1) * per] = True
+            r0 += n
+    return str(kind), mask
+
+
+def _like(s, data):
+    return stk.Matrix(s.size(), data, s.row_indices, s.column_indices, s.offsets, s.column_indices_t, s.offsets_t, s.block_offsets_t)
+
+
+@pytest.mark.parametrize("batch", range(5))
+def test_random_products_and_gradients_against_dense_fp32(batch):
+    for case in range(CASES_PER_TEST):
+        seed = 7000 + batch * CASES_PER_TEST + case
+        rng = np.random.RandomState(seed)
+        torch.manual_seed(seed)
+        b = int(rng.choice([128, 128, 64]))
+        dtype = torch.bfloat16 if rng.rand() < 0.5 else torch.float16
+        kind, mask = _pattern(rng)
+        m, k = mask.shape[0] * b, mask.shape[1] * b
+        n = b * int(rng.choice([1, 2, 3, 4, 8, rng.randint(1, 12)]))
+        inner = b * int(rng.choice([1, 2, 4, 8, rng.randint(1, 12)]))
+        ta, tb = bool(rng.rand() < 0.5), bool(rng.rand() < 0.5)
+        idx32 = bool(rng.rand() < 0.2)
+        info = dict(seed=seed, blocking=b, dtype=str(dtype), pattern=kind, shape=(m, k), n=n, inner=inner, ta=ta, tb=tb, idx32=idx32)
+        dense_mask = torch.from_numpy(np.kron(mask, np.ones((b, b), dtype=np.float32))).to(DEV)
+        vals = (torch.randn(m, k, device=DEV) * 0.5).to(dtype) * dense_mask.to(dtype)
+        vals = torch.where((dense_mask > 0) & (vals == 0), torch.ones_like(vals), vals)   # to_sparse keeps every block of the mask
+        s = stk.ops.to_sparse(vals, b)
+        assert s.nnz == int(mask.sum()) * b * b, info
+        if idx32:
+            s = stk.Matrix(s.size(), s.data, s.row_indices.int(), s.column_indices.int(), s.offsets, s.column_indices_t.int(), s.offsets_t,
+                           s.block_offsets_t)
+        sd = vals.float()
+
+        def randn(*shape):
+            return (torch.randn(*shape, device=DEV) * 0.5).to(dtype)
+
+        def view(t, transposed):    # the same values, as a .t() view of a contiguous tensor or contiguous
+            return (t.t().contiguous().t() if transposed else t).detach().requires_grad_(True)
+
+        # dsd: op(S) rhs and its two gradients
+        rhs = randn(m if ta else k, n)
+        values, rhs_arg = s.data.detach().clone().requires_grad_(True), view(rhs, tb)
+        sm = _like(s, values)
+        out = stk.ops.dsd(sm.t() if ta else sm, rhs_arg)
+        _check("dsd", out, (sd.t() if ta else sd) @ rhs.float(), dtype, info)
+        dy = randn(*out.shape)
+        out.backward(dy)
+        _check("dsd: gradient of rhs", rhs_arg.grad, (sd if ta else sd.t()) @ dy.float(), dtype, info)
+        ds = (rhs.float() @ dy.float().t()) if ta else (dy.float() @ rhs.float().t())
+        _check("dsd: gradient of the values", stk.ops.to_dense(_like(s, values.grad)), ds * dense_mask, dtype, info)
+
+        # dds: lhs op(S) and its two gradients
+        lhs = randn(n, k if tb else m)
+        values, lhs_arg = s.data.detach().clone().requires_grad_(True), view(lhs, ta)
+        sm = _like(s, values)
+        out = stk.ops.dds(lhs_arg, sm.t() if tb else sm)
+        _check("dds", out, lhs.float() @ (sd.t() if tb else sd), dtype, info)
+        dy = randn(*out.shape)
+        out.backward(dy)
+        _check("dds: gradient of lhs", lhs_arg.grad, dy.float() @ (sd if tb else sd.t()), dtype, info)
+        ds = (dy.float().t() @ lhs.float()) if tb else (lhs.float().t() @ dy.float())
+        _check("dds: gradient of the values", stk.ops.to_dense(_like(s, values.grad)), ds * dense_mask, dtype, info)
+
+        # sdd: lhs rhs on the pattern and its two gradients
+        lhs, rhs = randn(m, inner), randn(inner, k)
+        lhs_arg, rhs_arg = view(lhs, ta), view(rhs, tb)
+        out = stk.ops.sdd(lhs_arg, rhs_arg, s)
+        _check("sdd", stk.ops.to_dense(out), (lhs.float() @ rhs.float()) * dense_mask, dtype, info)
+        dvalues = randn(*out.data.shape)
+        out.data.backward(dvalues)
+        ds = stk.ops.to_dense(_like(s, dvalues)).float()
+        _check("sdd: gradient of lhs", lhs_arg.grad, ds @ rhs.float().t(), dtype, info)
+        _check("sdd: gradient of rhs", rhs_arg.grad, lhs.float().t() @ ds, dtype, info)
