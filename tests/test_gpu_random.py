@@ -119,3 +119,51 @@ def test_random_products_and_gradients_against_dense_fp32(batch):
         ds = stk.ops.to_dense(_like(s, dvalues)).float()
         _check("sdd: gradient of lhs", lhs_arg.grad, ds @ rhs.float().t(), dtype, info)
         _check("sdd: gradient of rhs", rhs_arg.grad, lhs.float().t() @ ds, dtype, info)
+
+
+def _same(name, got, want, info):
+    got = got.cpu().numpy() if torch.is_tensor(got) else np.asarray(got)
+    assert got.shape == np.asarray(want).shape and np.array_equal(got, want), (name, info)
+
+
+@pytest.mark.parametrize("batch", range(3))
+def test_random_routings_and_formats_bit_exact_against_the_oracle(batch):
+    # the integer paths: routing, the row copy into the padded layout, the dMoE topology of that routing, and
+    # to_sparse / transpose metadata / row_indices / to_dense on a random pattern, bit for bit against numpy
+    from oracle import stk_oracle as O
+    meta = ("offsets", "row_indices", "column_indices", "offsets_t", "column_indices_t", "block_offsets_t")
+    for case in range(25):
+        seed = 9000 + 25 * batch + case
+        rng = np.random.RandomState(seed)
+        tokens = int(rng.choice([1, 7, 100, 1000, 5000, rng.randint(1, 20000)]))
+        top_k = int(rng.choice([1, 1, 2, 2, 4, 3]))
+        experts = int(rng.choice([1, 2, 8, 64, 100, rng.randint(max(top_k, 1), 300)]))
+        blocking = int(rng.choice([8, 64, 128]))
+        skew = float(rng.choice([0.0, 1.2, 3.0]))
+        p = np.arange(1, experts + 1, dtype=np.float64) ** -skew
+        top = rng.choice(experts, size=(tokens, top_k), p=p / p.sum()).astype(np.int32)
+        info = dict(seed=seed, tokens=tokens, top_k=top_k, experts=experts, blocking=blocking, skew=skew)
+        want = O.route(top, experts, blocking)
+        r = stk.ops.route(torch.from_numpy(top).to(DEV), experts, blocking)
+        for f in want._fields:
+            _same("route " + f, getattr(r, f), getattr(want, f), info)
+        x = torch.randn(tokens, 8 * int(rng.randint(1, 40)), generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
+        _same("gather", stk.ops.padded_gather(x.to(DEV), r).float(), O.padded_gather(x.float().numpy(), want.row_slots, top_k), info)
+        if blocking >= 64 and experts <= 64:
+            per = int(rng.choice([1, 2, 4]))
+            t = stk.ops.dmoe_topology(r.padded_bins, blocking, int(want.padded_bins[-1]) // blocking, per, dtype=torch.bfloat16)
+            wt = O.dmoe_topology(np.diff(np.concatenate([[0], want.bins])), per * blocking, blocking)
+            for f in meta:
+                _same("dmoe_topology " + f, getattr(t, f), getattr(wt, f), info)
+        b = int(rng.choice([1, 2, 16, 64, 128]))
+        br, bc = int(rng.randint(1, 60)), int(rng.randint(1, 60))
+        mask = rng.rand(br, bc) < rng.choice([0.0, 0.05, 0.3, 0.9])
+        xd = (np.kron(mask, np.ones((b, b))) * rng.randn(br * b, bc * b)).astype(np.float16)
+        info = dict(seed=seed, blocking=b, block_rows=br, block_cols=bc)
+        s = stk.ops.to_sparse(torch.from_numpy(xd).to(DEV), b)
+        wd, wt = O.to_sparse(xd, b)
+        _same("to_sparse values", s.data, wd, info)
+        for f in meta:
+            _same("to_sparse " + f, getattr(s, f), getattr(wt, f), info)
+        _same("to_dense", stk.ops.to_dense(s), xd, info)
+        _same("row_indices", stk.ops.row_indices(s.size(), s.data, s.offsets, s.column_indices), wt.row_indices, info)
