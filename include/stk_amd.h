@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 12
+#define STK_AMD_ABI_VERSION 13
 
 /* status codes */
 #define STK_OK 0
@@ -240,6 +240,23 @@ int stk_dsd_dds(int64_t m, int64_t k,
                 const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
                 int64_t n_dsd, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, void* out_dsd, int64_t out_dsd_stride,
                 int64_t m_dds, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k, void* out_dds, int64_t out_dds_stride,
+                int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
+
+/*
+ * The same pair for a sampled product whose rhs was a .t() view of a row-major [k, n_t'] tensor (weights stored one
+ * row per output feature): the gradient with respect to that tensor is wanted in its own layout,
+ *   out   [m, n]    = S [m, k] * rhs [k, n]            the gradient with respect to lhs (rhs here = the row-major tensor)
+ *   out_t [k, n_t]  = S^T [k, m] * rhs_t [m, n_t]      the gradient with respect to the row-major tensor (rhs_t here = lhs there)
+ * two dsd products on the same values, which SDD.backward (stk/backend/sputnik.py:274-299) issues as two backend
+ * calls.  With blocking 128, a plan, row-major rhs and rhs_t and n, n_t multiples of 256 they run as one grid (the tiles
+ * of the first, then of the second); any other case runs stk_dsd twice (without a workspace).  Either way the results
+ * are those of the two stk_dsd calls without a workspace, bit for bit.
+ */
+int stk_dsd_dsd(int64_t m, int64_t k,
+                const void* data, const int32_t* offsets, const void* column_indices,
+                const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                int64_t n, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, void* out, int64_t out_stride,
+                int64_t n_t, const void* rhs_t, int64_t rhs_t_stride_k, int64_t rhs_t_stride_n, void* out_t, int64_t out_t_stride,
                 int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream);
 
 /*

@@ -11,7 +11,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
 STK_F16, STK_BF16 = 0, 1
 STK_I16, STK_I32 = 0, 1
@@ -34,6 +34,8 @@ SIGNATURES = {
     "stk_dsd": (_int, [_i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _int, _p, _p, _i64, _p]),
     "stk_dds": (_int, [_i64, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _p, _int, _p, _i64, _i64, _int, _int, _int, _p, _p]),
     "stk_dsd_dds": (_int, [_i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64,
+                           _i64, _int, _int, _int, _p, _p]),
+    "stk_dsd_dsd": (_int, [_i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64,
                            _i64, _int, _int, _int, _p, _p]),
     "stk_sdd_dsd": (_int, [_i64, _i64, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _p, _i64, _i64, _i64, _p,
                            _p, _int, _i64, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _int, _p, _p]),

@@ -68,7 +68,7 @@ def _run_sdd(lhs, rhs, sp):
 # fill the compute units that the other leaves idle in its last round.
 OVERLAP_GRADIENTS = True
 _side_streams = {}
-# Both gradients of sdd (stk_dsd_dds) and of dsd (stk_sdd_dsd) in one launch each where the operands' layouts allow it,
+# Both gradients of sdd (stk_dsd_dds, stk_dsd_dsd) and of dsd (stk_sdd_dsd) in one launch each where the operands' layouts allow it,
 # instead of two launches side by side; the same results.
 JOINT_GRADIENTS = True
 
@@ -193,6 +193,13 @@ def _sdd_operand_gradients(ctx, lhs, rhs, sp, ds):
         drhs = torch.empty((lhs.size(1), sp.shape[1]), dtype=rhs.dtype, device=rhs.device)
         backend.dsd_dds(sp.shape, ds, *sp.meta, rhs.t(), dlhs, lhs.t(), drhs)
         return dlhs, drhs
+    if JOINT_GRADIENTS and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and rhs_is_view:
+        # rhs is a .t() view of a row-major tensor, whose gradient is dS^T lhs: two dsd on the same dS, one call
+        base = rhs.t()
+        dlhs = torch.empty((sp.shape[0], rhs.size(0)), dtype=lhs.dtype, device=lhs.device)
+        dbase = torch.empty((sp.shape[1], lhs.size(1)), dtype=rhs.dtype, device=rhs.device)
+        backend.dsd_dsd(sp.shape, ds, *sp.meta, base, dlhs, lhs, dbase)
+        return dlhs, dbase.t()
     if ctx.needs_input_grad[0]:
         if lhs_is_view:
             want_lhs = lambda: _run_dds(rhs, sp, ds, True)              # rhs dS^T, returned transposed

@@ -387,6 +387,31 @@ def dsd_dds(shape, data, offsets, row_indices, column_indices, offsets_t, column
             data.shape[0], b, _value_dtype(data), _INDEX_DTYPES[ci.dtype], plan.data_ptr() if plan is not None else None, _stream()))
 
 
+def dsd_dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t, rhs, out, rhs_t, out_t):
+    """out = sparse @ rhs and out_t = sparse^T @ rhs_t for one sparse operand [m, k] = `shape`, in one launch where the
+    layouts allow it (the two gradients of an sdd whose rhs was a .t() view, stk/backend/sputnik.py:274-299); otherwise
+    the two products one after the other.  The results are those of two dsd calls without the workspace, bit for bit."""
+    _need_gpu(data, rhs, rhs_t, out, out_t)
+    m, k = shape
+    assert rhs.shape[0] == k and rhs_t.shape[0] == m, "incompatible dimensions"
+    b = _blocking(data)
+    _validate_matmul_dims(m, k, rhs.shape[1], b)
+    _validate_matmul_dims(k, m, rhs_t.shape[1], b)
+    rhs, rhs_t = _dense_operand(rhs), _dense_operand(rhs_t)
+    data = data.detach()
+    assert data.is_contiguous() and out.stride(1) == 1 and out_t.stride(1) == 1
+    assert data.dtype == rhs.dtype == rhs_t.dtype == out.dtype == out_t.dtype
+    ci, cit = _index(column_indices), _index(column_indices_t)
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b) if FUSION and b in (64, 128) and data.shape[0] > 0 else None
+    with _on_device(out.device):
+        _lib.check(_lib.load().stk_dsd_dsd(
+            m, k, data.data_ptr(), _offsets(offsets).data_ptr(), ci.data_ptr(),
+            _offsets(offsets_t).data_ptr(), cit.data_ptr(), _offsets(block_offsets_t).data_ptr(),
+            rhs.shape[1], rhs.data_ptr(), rhs.stride(0), rhs.stride(1), out.data_ptr(), out.stride(0),
+            rhs_t.shape[1], rhs_t.data_ptr(), rhs_t.stride(0), rhs_t.stride(1), out_t.data_ptr(), out_t.stride(0),
+            data.shape[0], b, _value_dtype(data), _INDEX_DTYPES[ci.dtype], plan.data_ptr() if plan is not None else None, _stream()))
+
+
 def sdd_dsd(shape, lhs, rhs_sdd, out_sdd, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t,
             transpose_a, rhs_dsd, out_dsd):
     """out_sdd = lhs @ rhs_sdd on the topology [m, n] = `shape` and out_dsd = op(sparse) @ rhs_dsd for the values `data` on the

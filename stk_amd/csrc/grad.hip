@@ -1,4 +1,4 @@
-// stk_dsd_dds and stk_sdd_dsd: the two gradients of a product in one launch.
+// stk_dsd_dds, stk_dsd_dsd and stk_sdd_dsd: the two gradients of a product in one launch.
 //
 // The backward pass of S = lhs x rhs (sampled on a topology) computes dS x rhs^T, a dsd, and lhs^T x dS, a dds,
 // from the same sparse values dS.  Here both run as one grid: first the tiles of the dsd (long walks along a block
@@ -6,6 +6,10 @@
 // units that the last long ones leave idle, and the blocks of dS that the dsd brought into the caches are still
 // on their way through them when the dds asks for them.  The tiles are the ones of stk_dsd and stk_dds
 // (dsd_tile.h, dds_tile.h), so the results are theirs bit for bit.
+//
+// When rhs reached the sampled product as a .t() view of a row-major [n, k] tensor (weights stored one row per output
+// feature), the second gradient is wanted in that tensor's layout: dS^T x lhs, a dsd on the transposed dS.
+// stk_dsd_dsd runs that pair the same way, the long row walks first, the short column walks behind them.
 //
 // The backward pass of y = op(S) x rhs computes dy x rhs^T on the topology, an sdd, and op(S)^T x dy, a dsd, from
 // the same dy.  stk_sdd_dsd runs them as one grid in the same way: the tiles of the sdd, which contract over all
@@ -61,6 +65,36 @@ static void launch_dsd_dds(const DsdArgs& d, const PlanLists& rows, const DdsArg
   // upper bound: every line a tile of its own in both products
   const int grid = d.block_rows * (d.n / DsdFused::TN) + s.block_cols * (s.m / DdsFused::TM);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, d, rows, s, cols);
+}
+
+// 128-blocks, eight wavefronts: the tiles of S x rhs from the plan's lists of block rows, then the tiles of
+// S^T x rhs_t from its lists of block columns, both as in dsd_fused_kernel.
+template <class Fused, class Triple, class Single, class FusedT, class TripleT, class SingleT>
+__global__ __launch_bounds__(512, 2) void dsd_dsd_kernel(DsdArgs d, PlanLists rows, DsdArgs t, PlanLists cols) {
+  extern __shared__ __align__(16) char smem[];
+  int bid = blockIdx.x;
+  if (dsd_plan_tile<Fused, Triple, Single, false>(d, rows, bid, smem)) return;
+  dsd_plan_tile<FusedT, TripleT, SingleT, true>(t, cols, bid, smem);
+}
+
+// Both dense operands row-major.  STREAM / STREAM_T: the rhs panels of the product are read about once.
+template <bool BF16, bool STREAM, bool STREAM_T>
+static void launch_dsd_dsd(const DsdArgs& d, const PlanLists& rows, const DsdArgs& t, const PlanLists& cols, hipStream_t stream) {
+  // the configurations of launch_dsd for the plain and for the transposed sparse operand
+  using Fused = TileCfg<4, 2, 2, 4, 1, 2, 2, true, false, BF16, STK_DSD_KT, STK_DSD_STAGES, false, STREAM>;
+  using Single = TileCfg<2, 4, 2, 2, 1, 1, 2, true, false, BF16, STK_DSD_KT, STK_DSD_STAGES, false, STREAM>;
+  using Triple = TileCfg<4, 2, 3, 2, 1, 3, 1, true, false, BF16, STK_DSD_KT, STK_DSD_STAGES, false, STREAM>;
+  using FusedT = TileCfg<4, 2, 2, 4, 1, 2, 2, false, false, BF16, STK_DSD_T_KT, STK_DSD_T_STAGES, false, STREAM_T>;
+  using SingleT = TileCfg<2, 4, 2, 2, 1, 1, 2, false, false, BF16, STK_DSD_T_KT, STK_DSD_T_STAGES, false, STREAM_T>;
+  using TripleT = TileCfg<4, 2, 3, 2, 1, 3, 1, false, false, BF16, STK_DSD_T_KT, STK_DSD_T_STAGES, false, STREAM_T>;
+  constexpr int lds = largest({Fused::kSmemBytes, Single::kSmemBytes, Triple::kSmemBytes, FusedT::kSmemBytes, SingleT::kSmemBytes,
+                               TripleT::kSmemBytes});
+  auto kernel = &dsd_dsd_kernel<Fused, Triple, Single, FusedT, TripleT, SingleT>;
+  static const int once = (set_lds_limit(kernel, lds), 0);
+  (void)once;
+  // upper bound: every line a tile of its own in both products
+  const int grid = d.block_rows * (d.n / Fused::TN) + t.block_rows * (t.n / FusedT::TN);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, d, rows, t, cols);
 }
 
 // 128-blocks, eight wavefronts: the tiles of the sdd from the plan's tile list as in sdd_fused_kernel, then the tiles
@@ -138,6 +172,43 @@ extern "C" int stk_dsd_dds(int64_t m, int64_t k,
     else launch_dsd_dds<false, false>(dsd.g, dsd.lists, dds.g, dds.lists, s);
   }
   return check_launch("stk_dsd_dds");
+}
+
+extern "C" int stk_dsd_dsd(int64_t m, int64_t k,
+                           const void* data, const int32_t* offsets, const void* column_indices,
+                           const int32_t* offsets_t, const void* column_indices_t, const int32_t* block_offsets_t,
+                           int64_t n, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, void* out, int64_t out_stride,
+                           int64_t n_t, const void* rhs_t, int64_t rhs_t_stride_k, int64_t rhs_t_stride_n, void* out_t, int64_t out_t_stride,
+                           int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
+  using namespace stk;
+  DsdProblem plain, transposed;
+  int rc = dsd_problem("stk_dsd_dsd", m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k,
+                       rhs_stride_n, out, out_stride, nnz, blocking, dtype, index_dtype, plan, &plain);
+  if (rc != STK_OK) return rc;
+  rc = dsd_problem("stk_dsd_dsd", k, m, n_t, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 1, rhs_t, rhs_t_stride_k,
+                   rhs_t_stride_n, out_t, out_t_stride, nnz, blocking, dtype, index_dtype, plan, &transposed);
+  if (rc != STK_OK) return rc;
+  // (the grid of the one launch - an upper bound on the tiles of both products - must be a 32-bit count)
+  const bool together = plan && blocking == 128 && nnz > 0 && !plain.empty && !transposed.empty && !plain.bk && !transposed.bk && n % 256 == 0 &&
+                        n_t % 256 == 0 && !plain.g.small && !transposed.g.small &&
+                        (int64_t)plain.g.block_rows * (n / 256) + (int64_t)transposed.g.block_rows * (n_t / 256) <= INT32_MAX;
+  if (!together) {
+    // shapes or layouts the joint launch has no tiles for: the two products one after the other
+    rc = stk_dsd(m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k, rhs_stride_n, out,
+                 out_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+    if (rc != STK_OK) return rc;
+    return stk_dsd(k, m, n_t, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 1, rhs_t, rhs_t_stride_k, rhs_t_stride_n,
+                   out_t, out_t_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define STK_DSD_DSD_CASE(BF, ST, STT)                                                                            \
+  if ((dtype == STK_BF16) == BF && plain.stream_rhs == ST && transposed.stream_rhs == STT) {                      \
+    launch_dsd_dsd<BF, ST, STT>(plain.g, plain.lists, transposed.g, transposed.lists, s);                         \
+    return check_launch("stk_dsd_dsd");                                                                           \
+  }
+  STK_DSD_DSD_CASE(true, true, true) STK_DSD_DSD_CASE(true, true, false) STK_DSD_DSD_CASE(true, false, true) STK_DSD_DSD_CASE(true, false, false)
+  STK_DSD_DSD_CASE(false, true, true) STK_DSD_DSD_CASE(false, true, false) STK_DSD_DSD_CASE(false, false, true) STK_DSD_DSD_CASE(false, false, false)
+  return fail(STK_ERR_UNSUPPORTED, "stk_dsd_dsd: no kernel for this configuration");
 }
 
 extern "C" int stk_sdd_dsd(int64_t m, int64_t n,

@@ -538,6 +538,37 @@ def test_both_gradients_of_sdd_in_one_call(dtype, blocking, hidden, ffn, tokens,
     assert torch.equal(grads[True][0], dx) and torch.equal(grads[True][1], dw1)
 
 
+@pytest.mark.parametrize("dtype,blocking,hidden,ffn,tokens", _JOINT_CASES)
+def test_both_gradients_of_sdd_with_a_transposed_rhs_in_one_call(dtype, blocking, hidden, ffn, tokens, monkeypatch):
+    # stk_dsd_dsd: for S = x W^T with W stored [columns of S, hidden], dS W and dS^T x from one call (one launch for
+    # 128-blocks with enough work; otherwise the two products one after the other) against the oracle's dsd, and bit for
+    # bit against the separate launches
+    from stk_amd.backend import autograd, hip_kernels
+    monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
+    topo, tm, x, w1, w2 = _dmoe_case(np.array(tokens), hidden, ffn, blocking, dtype, 35)
+    w = w2                                                   # [columns of S, hidden], row-major
+    g = torch.Generator().manual_seed(36)
+    ds = (torch.randn(tm.data.shape, generator=g) * 0.05).to(dtype).to(DEV)
+    dsm = stk.Matrix(tm.size(), ds, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
+    rows, cols = tm.size()
+    dx = torch.full((rows, hidden), float("nan"), dtype=dtype, device=DEV)
+    dw = torch.full((cols, hidden), float("nan"), dtype=dtype, device=DEV)
+    hip_kernels.dsd_dsd(tm.size(), ds, tm.offsets, tm.row_indices, tm.column_indices, tm.offsets_t, tm.column_indices_t, tm.block_offsets_t,
+                        w, dx, x, dw)
+    U.assert_close(dx, O.dsd(topo.shape, U.np32(ds), topo, False, U.np32(w)), dtype, "dS W")
+    U.assert_close(dw, O.dsd((cols, rows), U.np32(ds), topo, True, U.np32(x)), dtype, "dS^T x")
+    assert torch.equal(dx, stk.ops.dsd(dsm, w)) and torch.equal(dw, stk.ops.dsd(dsm.t(), x))
+    # through autograd: the gradients of sdd(x, W^T) with the joint call and with two launches
+    grads = {}
+    for joint in (True, False):
+        monkeypatch.setattr(autograd, "JOINT_GRADIENTS", joint)
+        xs, ws = x.detach().clone().requires_grad_(True), w.detach().clone().requires_grad_(True)
+        stk.ops.sdd(xs, ws.t(), tm).data.backward(ds)
+        grads[joint] = (xs.grad, ws.grad)
+    assert torch.equal(grads[True][0], grads[False][0]) and torch.equal(grads[True][1], grads[False][1])
+    assert torch.equal(grads[True][0], dx) and torch.equal(grads[True][1], dw)
+
+
 @pytest.mark.parametrize("transpose_a", [False, True])
 @pytest.mark.parametrize("dtype,blocking,hidden,ffn,tokens", _JOINT_CASES)
 def test_both_gradients_of_dsd_in_one_call(dtype, blocking, hidden, ffn, tokens, transpose_a, monkeypatch):
