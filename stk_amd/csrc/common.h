@@ -79,10 +79,17 @@ __host__ __device__ inline size_t plan_list_offset(int64_t block_rows, int64_t b
 // operand has 256 (t + 1) columns (wider: as 256 * 16).  Byte kSpreadHint: 1 when equal eighths of the lines hold
 // unequal numbers of blocks (read by the dsd with a sliced last round, see xcd_share()).
 // Bytes kGroupHint .. kGroupHint + kPlanLists - 1: for each list, how many consecutive entries go to one compute die
-// at a time (see xcd_item()).
+// at a time (see xcd_item()).  Bytes kStripeHint, kStripeHint + 1 (plans for 128-blocks): from how many 128-wide tiles
+// of the dense operand on the launches that give every line a tile of its own deal their tiles to the compute dies by
+// stripes of the dense operand instead of by lines (0: never), for the lists of threes / pairs / lone lines and for the
+// lists of pairs / lone lines.  By lines, a die fetches the dense panel of every block of its lines (G panels in all, G =
+// the blocks of one line per group of identical lines) and every sparse block once; by stripes, a die fetches its
+// stripe of every panel (K panels in all, K = the lines of the other direction) and every sparse block: stripes move
+// less when 1024 nnz + K w < 128 nnz + G w for a dense operand of w 256-byte columns, w > 896 nnz / (G - K).
 constexpr int kTailSliceColumns = 16;
 constexpr int kSpreadHint = 16;
 constexpr int kGroupHint = 17;
+constexpr int kStripeHint = 22;
 constexpr int kPlanHintBytes = 32;
 constexpr int kMaxTailSlices = 4;
 __host__ __device__ inline size_t plan_slices_offset(int64_t block_rows, int64_t block_cols) {
@@ -101,6 +108,12 @@ struct PlanLists {
     const int at = kGroupHint + k;
     const int e = (((words_t)(uintptr_t)hints)[at >> 2] >> (8 * (at & 3))) & 0xff;
     return e > 0 ? e : 1;
+  }
+  // 128-wide tiles of the dense operand from which on a launch over lone lines deals by stripes; 0: never
+  __device__ int stripe_from(bool tall) const {
+    typedef const __attribute__((address_space(4))) int32_t* words_t;
+    const int at = kStripeHint + (tall ? 0 : 1);
+    return (((words_t)(uintptr_t)hints)[at >> 2] >> (8 * (at & 3))) & 0xff;
   }
 };
 inline PlanLists plan_lists_of(const uint8_t* plan, int64_t block_rows, int64_t block_cols, bool columns) {

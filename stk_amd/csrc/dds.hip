@@ -28,7 +28,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dds_lines_kernel(DdsArgs g, 
   const int pairs = const_ints(plan.counts)[kPairs];
   const int tiles = (2 * pairs + const_ints(plan.counts)[kSingles]) * ntm;
   if ((int)blockIdx.x >= tiles) return;
-  const int item = xcd_grouped(blockIdx.x, tiles);
+  const int item = xcd_lines(blockIdx.x, tiles, ntm, plan.stripe_from(false));   // (by stripes of lhs rows when the columns share little)
   const int l = item / ntm;
   const int line = l < 2 * pairs ? const_ints(plan.list(kPairs))[l >> 1] + (l & 1) : const_ints(plan.list(kSingles))[l - 2 * pairs];
   dds_tile<Cfg, BLK, TRANS_B, true, 1>(g, line, (item % ntm) * Cfg::TM, smem);

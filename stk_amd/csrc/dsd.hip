@@ -20,7 +20,9 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_kernel(DsdArgs g) {
 
 // Every block row on its own (four wavefronts), in the order of the plan's lists: the rows of the pairs, of the
 // threes, then the lone rows longest first - for launches with little work per compute unit, where the order in
-// which the tiles start decides how evenly the units are loaded.
+// which the tiles start decides how evenly the units are loaded.  When the plan says that the rows share little
+// (a random pattern), every compute die takes a stripe of the dense operand's columns for all rows instead of all
+// columns for some rows, and fetches that stripe once (xcd_lines).
 template <class Cfg, int BLK, bool TRANS_A>
 __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_lines_kernel(DsdArgs g, PlanLists plan) {
   extern __shared__ __align__(16) char smem[];
@@ -28,7 +30,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_lines_kernel(DsdArgs g, 
   const int pairs = const_ints(plan.counts)[kTallPairs], triples = const_ints(plan.counts)[kTallTriples];
   const int tiles = (2 * pairs + 3 * triples + const_ints(plan.counts)[kTallSingles]) * ntn;
   if ((int)blockIdx.x >= tiles) return;
-  const int item = xcd_grouped(blockIdx.x, tiles);
+  const int item = xcd_lines(blockIdx.x, tiles, ntn, plan.stripe_from(true));
   int l = item / ntn, line;
   if (l < 2 * pairs) line = const_ints(plan.list(kTallPairs))[l >> 1] + (l & 1);
   else if ((l -= 2 * pairs) < 3 * triples) line = const_ints(plan.list(kTallTriples))[l / 3] + l % 3;

@@ -369,6 +369,7 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
     // quarter of a die's share of the list's blocks when they are as long as the first, the longest, entry - the
     // first group is the heaviest, and a die that gets too much of the launch in one piece holds it up - rounded
     // down to a power of two, between 1 and 32.
+    int blocks_of_groups[2] = {0, 0};  // (thread 0) blocks of one line per entry: lists of pairs / lone lines, lists with threes
     for (int kind = 0; kind < kPlanLists; kind++) {
       const int count = totals[kind];
       const int32_t* list = lists + 2 * kPlanLists + (cols ? kPlanLists * block_rows : 0) + kind * lines;
@@ -387,6 +388,21 @@ __global__ __launch_bounds__(1024) void plan_roles_kernel(const int32_t* __restr
           while (entries < 32 && 2 * entries <= fit) entries *= 2;
         }
         tail_slices[kGroupHint + kind] = (uint8_t)entries;
+        blocks_of_groups[kind >= kTallPairs ? 1 : 0] += total_blocks;
+      }
+    }
+    if (tid == 0) {
+      // from which width of the dense operand on stripes beat lines (kStripeHint); plans for 128-blocks only
+      const int64_t nnz = offs[lines];
+      const int others = cols ? block_rows : block_cols;
+      for (int family = 0; family < 2; family++) {
+        const int64_t saved = (int64_t)blocks_of_groups[family] - others;  // dense panels that stripes fetch fewer
+        int from = 0;
+        if (most == 2 && saved > 0) {
+          const int64_t tiles = (7 * nnz + saved - 1) / saved;  // 896 nnz / saved columns, in tiles of 128 columns
+          from = tiles > 255 ? 0 : (tiles < 1 ? 1 : (int)tiles);
+        }
+        tail_slices[kStripeHint + (family ? 0 : 1)] = (uint8_t)from;
       }
     }
     __syncthreads();

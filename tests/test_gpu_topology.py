@@ -271,6 +271,23 @@ def test_fusion_plan_roles(name):
                 while entries < 32 and 2 * entries <= fit:
                     entries *= 2
             assert int(h[17 + kind]) == entries, (d, kind, count)
+        # and from how many 128-wide tiles of the dense operand on the launches over single lines deal their tiles to
+        # the compute dies by stripes of the dense operand: ceil(7 nnz / (G - K)), G = the blocks of one line per list
+        # entry, K = the lines of the other direction (0: never; beyond 255: never); byte 22 for the lists with threes,
+        # byte 23 for the lists of pairs and lone lines
+        others = bc if d == 0 else br
+        for byte, kinds in ((22, (2, 3, 4)), (23, (0, 1))):
+            g_blocks = 0
+            for kind in kinds:
+                count = int(lists[5 * d + kind])
+                members = lists[base + kind * lines: base + kind * lines + count].tolist()
+                g_blocks += sum(int(offs[i + 1]) - int(offs[i]) for i in members)
+            saved = g_blocks - others
+            want = 0
+            if saved > 0:
+                want = max(1, -(-7 * int(offs[lines]) // saved))
+                want = 0 if want > 255 else want
+            assert int(h[byte]) == want, (d, byte, g_blocks, others)
     # in front: the tiles of sdd
     sdd = whole[:8 + 8 * max_tiles].view(np.int32)
     assert sdd[2:2 + 2 * sdd[0]].reshape(-1, 2).tolist() == _sdd_tiles(topo.offsets, topo.column_indices, 2, 2)
