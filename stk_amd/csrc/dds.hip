@@ -99,7 +99,8 @@ __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists 
   }
   bid -= pair_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
+    // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
+    const int item = xcd_lines(bid, single_tiles, ntm, (plan.stripe_from(false) + 1) >> 1);
     dds_tile<Single, 128, TRANS_B, true, 1>(g, const_ints(plan.list(kSingles))[item / ntm], (item % ntm) * Single::TM, smem);
   }
 }

@@ -266,7 +266,18 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
     return;
   }
   item -= triple_tiles;
-  const int i = xcd_grouped(item, single_tiles);  // (in order of length: no contiguous shares)
+  // (in order of length: no contiguous shares.)  When the plan says that the lone lines share little, the lines whose tiles all
+  // lie in the whole rounds, where a workgroup's id is its item, are dealt by stripes of the dense operand (xcd_lines; the
+  // list must start at a multiple of the eight dies, so that every line's tiles stay among themselves); what is left
+  // of the list is taken in order.
+  const int from = (plan.stripe_from(true) + 1) >> 1, lead = pair_tiles + triple_tiles;
+  int i;
+  if (from != 0 && ntn >= from && !(ntn & 7) && !(lead & 7)) {
+    const int striped = whole > lead ? (whole - lead) / ntn * ntn : 0;
+    i = item < striped ? xcd_lines(item, striped, ntn, from) : item;
+  } else {
+    i = xcd_grouped(item, single_tiles);
+  }
   dsd_slice<Single, TRANS_A, 1>(g, t, const_ints(plan.list(kTallSingles))[i / ntn], (i % ntn) * Single::TN, slice, slices, ordinal, smem, &flag);
 }
 

@@ -122,7 +122,8 @@ __device__ __forceinline__ bool dsd_plan_tile(const DsdArgs& g, const PlanLists&
   }
   bid -= triple_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
+    // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
+    const int item = xcd_lines(bid, single_tiles, ntn, (plan.stripe_from(true) + 1) >> 1);
     dsd_tile<Single, 128, TRANS_A, true, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
     return true;
   }

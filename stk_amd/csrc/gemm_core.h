@@ -802,13 +802,17 @@ __device__ __forceinline__ int xcd_item(int bid, int n, int per, int entries) {
 // The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
 // to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
 #ifndef STK_XCD_SDD_GROUP
-// Tiles of a launch that gives every line a tile of its own for each of `per` tiles of the dense operand (item = line
-// index * per + dense tile).  From `stripe_from` dense tiles on (0: never; the plan's hint) and when they divide by the
-// eight dies, die d takes the dense tiles [d per / 8, (d + 1) per / 8) of every line, in the order of the lines: it then
-// fetches its stripe of the dense operand once, whichever lines need it.  Otherwise groups of neighbouring items.
+// Tiles of a list of single lines, `per` tiles of the dense operand for each line (item = line index * per + dense
+// tile); bid counts from the list's first tile.  From `stripe_from` dense tiles on (0: never; the plan's hint) and
+// when they divide by the eight dies, die d takes the dense tiles [d per / 8, (d + 1) per / 8) of every line, in the
+// order of the lines: it then fetches its stripe of the dense operand once, whichever lines need it.  Otherwise
+// groups of neighbouring items.
 __device__ __forceinline__ int xcd_lines(int bid, int n, int per, int stripe_from) {
   if (stripe_from == 0 || per < stripe_from || (per & 7)) return xcd_grouped(bid, n);
-  const int share = per >> 3, die = bid & 7, local = bid >> 3;
+  // the workgroup's die, and how many of the list's tiles the die has taken before this one
+  const int id = blockIdx.x, first = id - bid, die = id & 7;
+  const int local = (id >> 3) - ((first + 7 - die) >> 3);
+  const int share = per >> 3;
   return (local / share) * per + die * share + local % share;
 }
 #define STK_XCD_SDD_GROUP 8

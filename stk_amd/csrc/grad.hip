@@ -37,7 +37,8 @@ __global__ __launch_bounds__(512, 2) void dsd_dds_kernel(DsdArgs d, PlanLists ro
   }
   bid -= pair_tiles;
   if (bid < single_tiles) {
-    const int item = xcd_grouped(bid, single_tiles);  // (in order of length: no contiguous shares)
+    // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
+    const int item = xcd_lines(bid, single_tiles, ntm, (cols.stripe_from(false) + 1) >> 1);
     dds_tile<DdsSingle, 128, false, true, 1>(s, const_ints(cols.list(kSingles))[item / ntm], (item % ntm) * DdsSingle::TM, smem);
   }
 }
