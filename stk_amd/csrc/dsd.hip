@@ -50,13 +50,13 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void dsd_singles_kernel(DsdArgs g
 }
 
 // 64-blocks with a plan built for them, eight wavefronts: groups of four identical block rows as 256x256
-// tiles (a group of three runs on the same shape with its fourth row dropped), pairs as 128x256 tiles; the dense
+// tiles, groups of three as 192x256 tiles, pairs as 128x256 tiles; the dense
 // operand is then read once per 256 or 128 rows instead of once per 64.  Lone rows are left to
 // dsd_singles_kernel.  The grid is an upper bound; the surplus leaves at once.
-template <class Quad, class Pair, bool TRANS_A>
+template <class Quad, class Pair, class Three, bool TRANS_A>
 __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanLists plan) {
   extern __shared__ __align__(16) char smem[];
-  static_assert(Quad::TN == Pair::TN, "same column tiling");
+  static_assert(Quad::TN == Pair::TN && Quad::TN == Three::TN, "same column tiling");
   const int ntn = g.n / Quad::TN;
   const int quad_tiles = const_ints(plan.counts)[kPairs] * ntn, triple_tiles = const_ints(plan.counts)[kTallTriples] * ntn;
   const int pair_tiles = const_ints(plan.counts)[kTallPairs] * ntn;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanList
   bid -= quad_tiles;
   if (bid < triple_tiles) {
     const int item = xcd_item(bid, triple_tiles, ntn, plan.group(kTallTriples));
-    dsd_tile<Quad, 64, TRANS_A, true, 4>(g, const_ints(plan.list(kTallTriples))[item / ntn], (item % ntn) * Quad::TN, smem, 3);
+    dsd_tile<Three, 64, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / ntn], (item % ntn) * Three::TN, smem);
   }
 }
 
@@ -342,11 +342,14 @@ static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* 
       // two), then the lone rows one per four-wave workgroup; both grids are upper bounds
       using Quad = TileCfg<4, 2, 2, 4, 1, 4, 2, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
       using Pair = TileCfg<2, 4, 2, 2, 1, 2, 2, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
+      // 2x4 wavefronts of 96x64 over three block rows: a group of three on a tile of its own size
+      using Three = TileCfg<2, 4, 3, 2, 1, 3, 2, !TRANS_A, BK, BF16, 64, 2, false, STREAM>;
       constexpr int lds = Quad::kSmemBytes > Pair::kSmemBytes ? Quad::kSmemBytes : Pair::kSmemBytes;
-      static const int once = (set_lds_limit(&dsd_fused64_kernel<Quad, Pair, TRANS_A>, lds), set_lds_limit(&dsd_singles_kernel<Dma, 64, TRANS_A, true>, Dma::kSmemBytes), 0);
+      static_assert(Three::kSmemBytes <= lds, "the tile of three block rows fits where the tile of four does");
+      static const int once = (set_lds_limit(&dsd_fused64_kernel<Quad, Pair, Three, TRANS_A>, lds), set_lds_limit(&dsd_singles_kernel<Dma, 64, TRANS_A, true>, Dma::kSmemBytes), 0);
       (void)once;
       const int ntn = g.n / 256;
-      hipLaunchKernelGGL((dsd_fused64_kernel<Quad, Pair, TRANS_A>), dim3((g.block_rows + 1) / 2 * ntn), dim3(512), lds, stream, g, plan);
+      hipLaunchKernelGGL((dsd_fused64_kernel<Quad, Pair, Three, TRANS_A>), dim3((g.block_rows + 1) / 2 * ntn), dim3(512), lds, stream, g, plan);
       hipLaunchKernelGGL((dsd_singles_kernel<Dma, 64, TRANS_A, true>), dim3(g.block_rows * ntn), dim3(Dma::kThreads), Dma::kSmemBytes, stream, g, plan);
       return;
     }
