@@ -361,6 +361,55 @@ def test_config2_uniform_random_all_variants():
         U.assert_close(stk.ops.sdd(lhs, rhs, s).data, O.sdd(lhs32, rhs32, topo), dtype, f"sdd {ta} {tb}")
 
 
+@pytest.mark.parametrize("slice_last_round", [True, False])
+def test_random_pattern_dealt_by_stripes_of_the_dense_operand(slice_last_round, monkeypatch):
+    # a random pattern with enough work for the eight-wave kernels and a dense operand of 2048 columns: the plan tells
+    # the launches to deal the lone lines to the compute dies by stripes of the dense operand (in the dsd with a sliced
+    # last round: the lines of its whole rounds).  A few repeated rows make pairs, whose tiles lie in front of the lone
+    # lines' in the grid.  Against the oracle, bit for bit against the launches without a plan (no slicing), and through
+    # the joint launch of an sdd and a dsd, where the list of lone lines starts anywhere in the grid.
+    from stk_amd.backend import hip_kernels
+    monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", slice_last_round)
+    dtype = torch.bfloat16
+    rng = np.random.RandomState(5)
+    mask = rng.rand(48, 40) < 0.5
+    mask[7] = mask[6]
+    mask[21] = mask[20]
+    mask[22] = mask[20]
+    dense = torch.from_numpy(np.kron(mask, np.ones((128, 128), dtype=np.float32)))
+    values = (torch.randn(dense.shape, generator=torch.Generator().manual_seed(5)) * 0.05).to(dtype) * dense.to(dtype)
+    s = stk.ops.to_sparse(torch.where((dense > 0) & (values == 0), torch.ones_like(values), values).to(DEV), 128)
+    topo = U.topo_of(s)
+    rows, cols = s.size()
+    g = torch.Generator().manual_seed(6)
+    b = (torch.randn(cols, 2048, generator=g) * 0.05).to(dtype).to(DEV)
+    bt = (torch.randn(rows, 2048, generator=g) * 0.05).to(dtype).to(DEV)
+    a = (torch.randn(2048, rows, generator=g) * 0.05).to(dtype).to(DEV)
+    plan = hip_kernels.fusion_plan(s.offsets, s.column_indices, s.offsets_t, s.column_indices_t).cpu().numpy()
+    br, bc, nnz = rows // 128, cols // 128, s.data.shape[0]
+    hints = plan[8 + 8 * ((nnz + br + 1) // 2) + (3 * (br + bc) + 3) // 4 * 4 + 4 * 5 * (2 + br + bc):]
+    assert 0 < hints[22] <= 16 and 0 < hints[32 + 23] <= 16, "the plan asks for stripes at this width"
+    data32 = U.np32(s.data)
+    got = {"dsd": stk.ops.dsd(s, b), "dsd t": stk.ops.dsd(s.t(), bt), "dds": stk.ops.dds(a, s), "dds t": stk.ops.dds(b.t(), s.t())}
+    U.assert_close(got["dsd"], O.dsd((rows, cols), data32, topo, False, U.np32(b)), dtype, "dsd")
+    U.assert_close(got["dsd t"], O.dsd((cols, rows), data32, topo, True, U.np32(bt)), dtype, "dsd t")
+    U.assert_close(got["dds"], O.dds(U.np32(a), (rows, cols), data32, topo, False), dtype, "dds")
+    U.assert_close(got["dds t"], O.dds(U.np32(b).T, (cols, rows), data32, topo, True), dtype, "dds t")
+    if not slice_last_round:
+        monkeypatch.setattr(hip_kernels, "FUSION", False)
+        plain = {"dsd": stk.ops.dsd(s, b), "dsd t": stk.ops.dsd(s.t(), bt), "dds": stk.ops.dds(a, s), "dds t": stk.ops.dds(b.t(), s.t())}
+        monkeypatch.setattr(hip_kernels, "FUSION", True)
+        for what in got:
+            assert torch.equal(got[what], plain[what]), what
+        dy = bt
+        ds = torch.empty_like(s.data)
+        drhs = torch.empty(cols, 2048, dtype=dtype, device=DEV)
+        meta = (s.offsets, s.row_indices, s.column_indices, s.offsets_t, s.column_indices_t, s.block_offsets_t)
+        w = (torch.randn(cols, 2048, generator=g) * 0.05).to(dtype).to(DEV)
+        hip_kernels.sdd_dsd(s.size(), dy, w.t(), ds, s.data, *meta, True, dy, drhs)
+        assert torch.equal(ds, stk.ops.sdd(dy, w.t(), s).data) and torch.equal(drhs, got["dsd t"])
+
+
 def _dmoe_case(tokens, hidden, ffn, blocking, dtype, seed):
     topo = O.dmoe_topology(tokens, ffn, blocking)
     g = torch.Generator().manual_seed(seed)
