@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
 ABI_VERSION = 13
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
-STK_F16, STK_BF16 = 0, 1
+STK_F16, STK_BF16, STK_F32 = 0, 1, 2
 STK_I16, STK_I32 = 0, 1
 
 _p, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t

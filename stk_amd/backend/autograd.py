@@ -84,7 +84,7 @@ def _side_stream(device):
 def _both(first, second, device):
     """first() and second() -> their results (None for a callable that is None), launched side by side when
     both are wanted.  Each callable launches one product and returns its freshly allocated output."""
-    if first is None or second is None or not OVERLAP_GRADIENTS:
+    if first is None or second is None or not OVERLAP_GRADIENTS or device.type != "cuda":
         return (first() if first is not None else None), (second() if second is not None else None)
     main = torch.cuda.current_stream(device)
     side = _side_stream(device)
@@ -121,7 +121,7 @@ class DSD(torch.autograd.Function):
         dy = _plain(dy)
         want_data = want_rhs = None
         rhs_is_view = _is_transposed_view(rhs)
-        if JOINT_GRADIENTS and ctx.needs_input_grad[1] and ctx.needs_input_grad[9] and not rhs_is_view:
+        if JOINT_GRADIENTS and dy.is_cuda and ctx.needs_input_grad[1] and ctx.needs_input_grad[9] and not rhs_is_view:
             # dy rhs^T on the pattern and op(S)^T dy read the same dy: one call (sputnik.py:131-155 makes two)
             ddata = torch.empty_like(data)
             drhs = torch.empty_like(rhs, memory_format=torch.contiguous_format)
@@ -187,13 +187,13 @@ def _sdd_operand_gradients(ctx, lhs, rhs, sp, ds):
     """Gradients of S = lhs rhs (on the pattern) with respect to lhs and rhs, given dS as the values `ds`."""
     want_lhs = want_rhs = None
     lhs_is_view, rhs_is_view = _is_transposed_view(lhs), _is_transposed_view(rhs)
-    if JOINT_GRADIENTS and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and not rhs_is_view:
+    if JOINT_GRADIENTS and ds.is_cuda and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and not rhs_is_view:
         # dS rhs^T and lhs^T dS read the same dS: one call (sputnik.py:274-299 makes two)
         dlhs = torch.empty((sp.shape[0], rhs.size(0)), dtype=lhs.dtype, device=lhs.device)
         drhs = torch.empty((lhs.size(1), sp.shape[1]), dtype=rhs.dtype, device=rhs.device)
         backend.dsd_dds(sp.shape, ds, *sp.meta, rhs.t(), dlhs, lhs.t(), drhs)
         return dlhs, drhs
-    if JOINT_GRADIENTS and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and rhs_is_view:
+    if JOINT_GRADIENTS and ds.is_cuda and ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and not lhs_is_view and rhs_is_view:
         # rhs is a .t() view of a row-major tensor, whose gradient is dS^T lhs: two dsd on the same dS, one call
         base = rhs.t()
         dlhs = torch.empty((sp.shape[0], rhs.size(0)), dtype=lhs.dtype, device=lhs.device)
@@ -302,11 +302,7 @@ class RowIndices(torch.autograd.Function):
     @staticmethod
     def forward(ctx, shape, data, offsets, column_indices):
         out = torch.empty(column_indices.shape, dtype=column_indices.dtype, device=column_indices.device)
-        if out.is_cuda:
-            backend.row_indices(shape, data, offsets, column_indices, out)
-        else:
-            from stk_amd.backend import host_format
-            host_format.row_indices(offsets, out)
+        backend.row_indices(shape, data, offsets, column_indices, out)
         return out
 
 

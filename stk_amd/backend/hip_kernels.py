@@ -7,18 +7,20 @@ same shape violations (:15-19, :243, :299, :351).  `transpose_meta`, `to_dense`
 and `to_sparse` are the device versions of stk/matrix.py:105-123 and
 stk/ops/matrix_ops.py:36-85.
 
-Everything here needs tensors on a ROCm device and launches on torch's current
-stream without synchronising (to_sparse reads one int back, as the reference's
-torch.nonzero does).  Nothing falls back to another implementation.
+Device tensors launch on torch's current stream without synchronising (to_sparse
+reads one int back, as the reference's torch.nonzero does); for them nothing falls
+back to another implementation.  Calls of the four reference functions whose tensors
+all live in host memory are handed to the host library (host_kernels), which is how
+the reference's plumbing configuration - products on CPU tensors - runs here.
 """
 import ctypes
 import threading
 
 import torch
 
-from stk_amd.backend import _lib
+from stk_amd.backend import _lib, host_kernels
 
-_VALUE_DTYPES = {torch.float16: _lib.STK_F16, torch.bfloat16: _lib.STK_BF16}
+_VALUE_DTYPES = {torch.float16: _lib.STK_F16, torch.bfloat16: _lib.STK_BF16, torch.float32: _lib.STK_F32}
 _INDEX_DTYPES = {torch.int16: _lib.STK_I16, torch.int32: _lib.STK_I32}
 
 
@@ -70,7 +72,7 @@ def _need_gpu(*tensors):
 
 def _value_dtype(t):
     if t.dtype not in _VALUE_DTYPES:
-        raise NotImplementedError(f"stk_amd: products need float16 or bfloat16 values, got {t.dtype}")
+        raise NotImplementedError(f"stk_amd: products need float16, bfloat16 or float32 values, got {t.dtype}")
     return _VALUE_DTYPES[t.dtype]
 
 
@@ -229,12 +231,16 @@ def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activa
     rounding, multiplies by `multiplier` ([nnz, b, b] values of a matrix with the same topology).
     No counterpart as one call in the reference, whose callers run the activation and
     stk.ops.mul (stk/ops/eltwise_ops.py:3-28) as passes of their own over the values."""
-    _need_gpu(lhs, rhs, out)
     assert lhs.shape[1] == rhs.shape[0], "incompatible dimensions"
     m, k = lhs.shape
     n = rhs.shape[1]
     b = _blocking(out)
     _validate_matmul_dims(m, k, n, b)
+    if not out.is_cuda:
+        if ACTIVATIONS.get(activation, 1) != 0 or multiplier is not None:
+            raise NotImplementedError("stk_amd: the fused store of sdd runs on a GPU only")
+        return host_kernels.sdd(lhs, rhs, shape, out, offsets, row_indices, column_indices)
+    _need_gpu(lhs, rhs, out)
     assert out.is_contiguous()
     if activation not in ACTIVATIONS:
         raise ValueError(f"unknown activation {activation!r}; one of {sorted(k for k in ACTIVATIONS if k)}")
@@ -282,6 +288,28 @@ def release_workspaces():
     _dsd_workspaces.clear()
 
 
+def _workspace_choice(capturing, entry_stream, handle):
+    """Which workspace a dsd launch on the stream `handle` takes.  `capturing`: a graph capture is under way on that
+    stream; `entry_stream`: handle of the stream that last used the device's shared workspace (None: there is none yet).
+      "private"  a buffer of the launch's own.  Every captured launch: its buffer comes out of the graph's memory pool, so
+                 replays - on whatever stream, next to whatever eager launches or other graphs - share counters and
+                 partial-tile slots with nobody.
+      "create"   no shared workspace yet: allocate it for this stream.
+      "shared"   the shared workspace, last used on this very stream: launches on one stream cannot overlap.
+      "wait"     the shared workspace after waiting for the stream that used it last."""
+    if capturing:
+        return "private"
+    if entry_stream is None:
+        return "create"
+    return "shared" if entry_stream == handle else "wait"
+
+
+def _new_workspace(device, nbytes, counters):
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    ws[:counters].zero_()   # (a fill kernel, also under capture; the slots behind the counters need no initial value)
+    return ws
+
+
 def _dsd_workspace(device, m, n, blocking):
     """Workspace of stk_dsd for this shape, or None: [counters | slots], the counters zero between launches."""
     if not SLICE_LAST_ROUND:
@@ -294,15 +322,16 @@ def _dsd_workspace(device, m, n, blocking):
     entry = _dsd_workspaces.get(key)
     counters = lib.stk_dsd_workspace_counter_bytes()
     nbytes = counters + DSD_WORKSPACE_SLOTS * lib.stk_dsd_workspace_slot_bytes()
-    if entry is None or entry[0].numel() != nbytes:
-        if _capture_id(device):
-            return None     # a buffer made inside a capture would belong to that graph: this launch runs uncut
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        ws[:counters].zero_()   # the slots behind the counters need no initial value
-        entry = _dsd_workspaces[key] = [ws, torch.cuda.current_stream(device)]
-    elif entry[1].cuda_stream != handle and not _capture_id(device):
-        # (a capture cannot wait for work outside it: replays of a graph with such a launch must not overlap other
-        # dsd launches of the device, which holds when they are issued to the stream those use)
+    if entry is not None and entry[0].numel() != nbytes:
+        entry = None
+    choice = _workspace_choice(_capture_id(device) != 0, None if entry is None else entry[1].cuda_stream, handle)
+    if choice == "private":
+        # zeroed by a fill kernel that is part of the graph; the memory goes back to the graph's pool when the
+        # caller drops it, where only later allocations of the same capture, which run behind this launch, reuse it
+        return _new_workspace(device, nbytes, counters)
+    if choice == "create":
+        entry = _dsd_workspaces[key] = [_new_workspace(device, nbytes, counters), torch.cuda.current_stream(device)]
+    elif choice == "wait":
         stream = torch.cuda.current_stream(device)
         stream.wait_stream(entry[1])   # launches that share a workspace must not overlap
         entry[1] = stream
@@ -312,12 +341,15 @@ def _dsd_workspace(device, m, n, blocking):
 def dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,
         block_offsets_t, transpose_a, rhs, out):
     """out = op(sparse) @ rhs; `shape` is the logical shape of the sparse operand."""
-    _need_gpu(data, rhs, out)
     assert shape[1] == rhs.shape[0], "incompatible dimensions"
     m, k = shape
     n = rhs.shape[1]
     b = _blocking(data)
     _validate_matmul_dims(m, k, n, b)
+    if not out.is_cuda:
+        return host_kernels.dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t,
+                                transpose_a, rhs, out)
+    _need_gpu(data, rhs, out)
     rhs = _dense_operand(rhs)
     data = data.detach()
     assert data.is_contiguous() and out.stride(1) == 1
@@ -341,12 +373,15 @@ def dsd(shape, data, offsets, row_indices, column_indices, offsets_t, column_ind
 def dds(lhs, shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,
         block_offsets_t, transpose_b, out):
     """out = lhs @ op(sparse); `shape` is the logical shape of the sparse operand."""
-    _need_gpu(data, lhs, out)
     assert lhs.shape[1] == shape[0], "incompatible dimensions"
     m, k = lhs.shape
     n = shape[1]
     b = _blocking(data)
     _validate_matmul_dims(m, k, n, b)
+    if not out.is_cuda:
+        return host_kernels.dds(lhs, shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t, block_offsets_t,
+                                transpose_b, out)
+    _need_gpu(data, lhs, out)
     lhs = _dense_operand(lhs)
     data = data.detach()
     assert data.is_contiguous() and out.stride(1) == 1
@@ -444,6 +479,8 @@ def sdd_dsd(shape, lhs, rhs_sdd, out_sdd, data, offsets, row_indices, column_ind
 
 def row_indices(shape, data, offsets, column_indices, out):
     """out[offsets[r]:offsets[r+1]] = r for every block row r."""
+    if not out.is_cuda:
+        return host_kernels.row_indices(shape, data, offsets, column_indices, out)
     _need_gpu(offsets, out)
     assert out.is_contiguous()
     offsets = _offsets(offsets)

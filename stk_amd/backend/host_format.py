@@ -3,15 +3,23 @@
 The reference builds its matrices on the host and moves them to the device
 afterwards (stk/ops/linear_ops_test.py:57-63, stk/random/random_ops.py:26-28),
 so `to_sparse`, `to_dense` and the transpose metadata must accept CPU tensors.
-These are the torch statements for that case.  Device tensors never come
-here: they go to the HIP kernels (stk_amd/backend/hip_kernels.py), and the
-matrix products have no host implementation at all.
+Values of 2 or 4 bytes with 16- or 32-bit indices - everything the reference's
+tests and the products use - go to the host library (host_kernels); what is left
+(other element widths, 64-bit indices) is handled by the torch statements below.
+Device tensors never come here: they go to the HIP kernels
+(stk_amd/backend/hip_kernels.py).
 """
 import torch
+
+from stk_amd.backend import host_kernels
+
+_NARROW = (torch.int16, torch.int32)
 
 
 def transpose_meta(size, data, row_indices, column_indices, offsets):
     """stk/matrix.py:105-123 with a stable sort (ascending block id inside a column)."""
+    if row_indices.dtype in _NARROW and row_indices.dtype == column_indices.dtype:
+        return host_kernels.transpose_meta(size, data, row_indices, column_indices, offsets)
     block_cols = size[1] // data.shape[1]
     order = torch.argsort(column_indices.to(torch.int64), stable=True)
     column_indices_t = row_indices[order]
@@ -29,6 +37,8 @@ def _blocked_view(x, blocking):
 
 def to_sparse(x, blocking, index_dtype=torch.int16):
     """stk/ops/matrix_ops.py:64-85: nonzero blocks in row-major order."""
+    if host_kernels.handles(x) and index_dtype in _NARROW:
+        return host_kernels.to_sparse(x, blocking, index_dtype)
     blocks = _blocked_view(x, blocking)
     nonzero = (blocks != 0).flatten(2).any(dim=2)
     nonzero |= torch.isnan(blocks).flatten(2).any(dim=2) if x.is_floating_point() else False
@@ -41,13 +51,9 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
 
 def to_dense(data, row_indices, column_indices, rows, cols):
     """stk/ops/matrix_ops.py:36-47: zeros, then every block copied to its place."""
+    if host_kernels.handles(data) and row_indices.dtype in _NARROW and row_indices.dtype == column_indices.dtype:
+        return host_kernels.to_dense(data, row_indices, column_indices, rows, cols)
     b = data.shape[-1]
     out = torch.zeros((rows, cols), dtype=data.dtype)
     _blocked_view(out, b)[row_indices.long(), column_indices.long()] = data
     return out
-
-
-def row_indices(offsets, out):
-    """stk/backend/triton_kernels.py:381-393."""
-    counts = (offsets[1:] - offsets[:-1]).long()
-    out.copy_(torch.repeat_interleave(torch.arange(counts.numel()), counts).to(out.dtype))

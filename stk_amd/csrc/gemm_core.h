@@ -799,9 +799,6 @@ __device__ __forceinline__ int xcd_item(int bid, int n, int per, int entries) {
   const int r = bid - base;
   return base + (r & 7) * group + (r >> 3);
 }
-// The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
-// to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
-#ifndef STK_XCD_SDD_GROUP
 // Tiles of a list of single lines, `per` tiles of the dense operand for each line (item = line index * per + dense
 // tile); bid counts from the list's first tile.  From `stripe_from` dense tiles on (0: never; the plan's hint) and
 // when they divide by the eight dies, die d takes the dense tiles [d per / 8, (d + 1) per / 8) of every line, in the
@@ -815,6 +812,9 @@ __device__ __forceinline__ int xcd_lines(int bid, int n, int per, int stripe_fro
   const int share = per >> 3;
   return (local / share) * per + die * share + local % share;
 }
+// The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
+// to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
+#ifndef STK_XCD_SDD_GROUP
 #define STK_XCD_SDD_GROUP 8
 #endif
 __device__ __forceinline__ int xcd_tile(int bid, int n) { return xcd_grouped<STK_XCD_SDD_GROUP>(bid, n); }

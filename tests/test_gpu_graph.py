@@ -113,7 +113,7 @@ def test_forward_and_backward_replay_from_a_graph():
 
 def test_a_plan_built_inside_a_capture_serves_that_capture_only(monkeypatch):
     # no call on this topology before the capture: its plan is built by the captured launches and exists only in the
-    # graph's replays, and there is no dsd workspace yet, so the captured dsd runs with its last round uncut
+    # graph's replays; the captured dsd cuts its last round with a workspace of the graph's own
     from stk_amd.backend import hip_kernels
     dtype = torch.bfloat16
     topo, tm, x, w1, w2, g = _case(1024, 4096, 128, dtype, 45)
@@ -132,15 +132,44 @@ def test_a_plan_built_inside_a_capture_serves_that_capture_only(monkeypatch):
     y_eager = stk.ops.dsd(h_eager, w2)
     h_other = stk.ops.sdd(x, w1, other)
     assert torch.equal(h_eager.data, h_other.data) and torch.equal(y_eager, stk.ops.dsd(h_other, w2))
-    monkeypatch.setattr(hip_kernels, "SLICE_LAST_ROUND", False)
-    y_uncut = stk.ops.dsd(h_other, w2)
+    eager_workspaces = dict(hip_kernels._dsd_workspaces)
     for replay in range(2):
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(h.data, h_eager.data) and torch.equal(y, y_uncut), replay
+        assert torch.equal(h.data, h_eager.data) and torch.equal(y, y_eager), replay
+    assert hip_kernels._dsd_workspaces == eager_workspaces          # the graph's workspace is not the device's
     with pytest.raises(RuntimeError, match="cannot be captured"):
         with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
             stk.ops.to_sparse(y, 128)
+
+
+def test_replays_beside_eager_launches_and_other_graphs_share_no_workspace():
+    # a captured dsd with a sliced last round owns its counters and partial-tile slots: replays on one stream next to
+    # eager launches and to the replays of a second graph on other streams all give the eager result
+    dtype = torch.bfloat16
+    topo, tm, x, w1, w2, g = _case(1024, 4096, 128, dtype, 49)
+    h = stk.ops.sdd(x, w1, tm)
+    want = stk.ops.dsd(h, w2)
+    want_t = stk.ops.dsd(h.t(), x)
+    torch.cuda.synchronize()
+    graphs, outs = [], []
+    for product in (lambda: stk.ops.dsd(h, w2), lambda: stk.ops.dsd(h.t(), x)):
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs.append(product())
+        graphs.append(graph)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for round_ in range(3):
+        for o in outs:
+            o.zero_()
+        torch.cuda.synchronize()
+        for graph, stream in zip(graphs, streams):
+            with torch.cuda.stream(stream):
+                graph.replay()
+        eager = stk.ops.dsd(h, w2)                      # on the default stream, with the device's workspace
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], want) and torch.equal(outs[1], want_t) and torch.equal(eager, want), round_
 
 
 def test_a_routed_layer_replays_from_a_graph_with_new_expert_choices():

@@ -80,14 +80,21 @@ def test_dsd_tail_slice_rule_matches_an_item_by_item_simulation(tiles, length):
     assert got == want, (got, want, ends)
 
 
-def test_products_refuse_host_tensors():
+def test_host_tensors_go_to_the_host_library_and_gpu_only_operations_refuse_them():
     m = stk.ops.to_sparse(torch.ones(128, 128, dtype=torch.float16), 128)
+    ones = torch.ones(128, 128, dtype=torch.float16)
+    assert torch.equal(stk.ops.dsd(m, ones), torch.full((128, 128), 128.0, dtype=torch.float16))
+    assert torch.equal(stk.ops.dds(ones, m), torch.full((128, 128), 128.0, dtype=torch.float16))
+    assert torch.equal(stk.ops.sdd(ones, ones, m).data, torch.full((1, 128, 128), 128.0, dtype=torch.float16))
+    # what exists on the GPU only says so
+    from stk_amd.backend import hip_kernels as hk
+    meta = (m.offsets, m.row_indices, m.column_indices, m.offsets_t, m.column_indices_t, m.block_offsets_t)
     with pytest.raises(RuntimeError, match="GPU"):
-        stk.ops.dsd(m, torch.ones(128, 128, dtype=torch.float16))
+        hk.dsd_dds((128, 128), m.data, *meta, ones, torch.empty_like(ones), ones, torch.empty_like(ones))
     with pytest.raises(RuntimeError, match="GPU"):
-        stk.ops.dds(torch.ones(128, 128, dtype=torch.float16), m)
+        stk.ops.route(torch.zeros(4, 1, dtype=torch.int32), 2, 128)
     with pytest.raises(RuntimeError, match="GPU"):
-        stk.ops.sdd(torch.ones(128, 128, dtype=torch.float16), torch.ones(128, 128, dtype=torch.float16), m)
+        stk.ops.dmoe_topology(torch.tensor([128], dtype=torch.int32), 128, 1, 1)
 
 
 def test_config1_known_answer_host_path():
@@ -196,6 +203,17 @@ def test_bench_rejects_what_it_does_not_measure():
         run = subprocess.run([sys.executable, os.path.join(root, "bench.py")] + flags, capture_output=True, text=True, timeout=300)
         assert run.returncode != 0
         assert text in run.stderr, run.stderr
+
+
+def test_dsd_workspace_choice():
+    # captured launches never touch the device's shared workspace; eager launches share it and serialise across streams
+    from stk_amd.backend.hip_kernels import _workspace_choice
+    assert _workspace_choice(True, None, 5) == "private"
+    assert _workspace_choice(True, 5, 5) == "private"       # even on the stream that owns the shared one: replays may run elsewhere
+    assert _workspace_choice(True, 7, 5) == "private"
+    assert _workspace_choice(False, None, 5) == "create"
+    assert _workspace_choice(False, 5, 5) == "shared"
+    assert _workspace_choice(False, 7, 5) == "wait"
 
 
 def test_fusion_plan_cache_is_tied_to_the_index_tensors_it_was_built_from():
