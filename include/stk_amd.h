@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 13
+#define STK_AMD_ABI_VERSION 14
 
 /* status codes */
 #define STK_OK 0
@@ -42,14 +42,16 @@ extern "C" {
 #define STK_ERR_WORKSPACE 4   /* workspace pointer missing or too small */
 
 /*
- * Element types of values.  The reference's launchers take whatever dtype the tensors have
- * (stk/backend/triton_kernels.py:250, 306, 358 pass the pointers on, float32 included); the products here compute
- * on 16-bit MFMA operands with fp32 accumulation and accept float16 and bfloat16 only.  Anything else is refused with
- * STK_ERR_UNSUPPORTED - nothing is converted silently: a float32 caller rounds its operands to one of the two types
- * itself and so chooses the precision it loses.  The format helpers (to_dense, to_sparse) take 2- and 4-byte elements.
+ * Element types of values.  The reference's launchers take whatever dtype the tensors have and accumulate in fp32
+ * (stk/backend/triton_kernels.py:250, 306, 358; ACC_TYPE :248).  Here float16 and bfloat16 run on the 16-bit MFMA tile
+ * engine; float32 runs on fp32 MFMA kernels of its own (one output block per workgroup, any element strides, no
+ * fusion plan or workspace - a compatibility path, not a tuned one).  All three accumulate in fp32 and round once.
+ * Anything else is refused with STK_ERR_UNSUPPORTED - nothing is converted silently.  The format helpers (to_dense,
+ * to_sparse) take 2- and 4-byte elements.
  */
 #define STK_F16 0
 #define STK_BF16 1
+#define STK_F32 2
 
 /* element types of row/column indices */
 #define STK_I16 0

@@ -56,6 +56,14 @@ inline int check_launch(const char* what) {
   return STK_OK;
 }
 
+// float32 values (fp32.hip): the products hand STK_F32 problems to these.
+int sdd_f32(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k, const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+            int64_t m, int64_t k, int64_t n, void* out, const void* row_indices, const void* column_indices, int64_t nnz,
+            int blocking, int index_dtype, int activation, const void* multiplier, hipStream_t stream);
+int walk_f32(bool sparse_lhs, const char* who, int64_t lines, int64_t free_extent, const void* data, const int32_t* walk_offsets,
+             const void* walk_positions, const int32_t* walk_blocks, bool line_major, const void* dense, int64_t dense_stride_free,
+             int64_t dense_stride_k, void* out, int64_t out_stride_m, int64_t nnz, int blocking, int index_dtype, hipStream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Layout of a fusion plan (see plan.hip).  First the tiles of stk_sdd (their size depends on the block

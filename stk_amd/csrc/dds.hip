@@ -228,6 +228,17 @@ extern "C" int stk_dds(int64_t m, int64_t k, int64_t n,
                        void* out, int64_t out_stride_m,
                        int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32) {
+    if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "stk_dds: negative size");
+    if (blocking > 0 && (k % blocking || n % blocking))
+      return fail(STK_ERR_DIMS, "incompatible dimensions: dense [%lld, %lld] x sparse [%lld, %lld] with blocking %d", (long long)m, (long long)k,
+                  (long long)k, (long long)n, blocking);
+    const bool tb = transpose_b != 0;
+    if (!tb && nnz > 0 && !block_offsets_t) return fail(STK_ERR_DIMS, "stk_dds: missing metadata pointer");
+    return walk_f32(false, "stk_dds", blocking > 0 ? n / blocking : 0, m, data, tb ? offsets : offsets_t, tb ? column_indices : column_indices_t,
+                    tb ? nullptr : block_offsets_t, tb, lhs, lhs_stride_m, lhs_stride_k, out, out_stride_m, nnz, blocking, index_dtype,
+                    static_cast<hipStream_t>(stream));
+  }
   DdsProblem problem;
   const int rc = dds_problem("stk_dds", m, k, n, lhs, lhs_stride_m, lhs_stride_k, data, offsets, column_indices, offsets_t, column_indices_t,
                              block_offsets_t, transpose_b, out, out_stride_m, nnz, blocking, dtype, index_dtype, plan, &problem);

@@ -428,6 +428,17 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
                        int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
                        void* workspace, int64_t workspace_bytes, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32) {
+    if (m < 0 || n < 0 || k < 0 || nnz < 0) return fail(STK_ERR_DIMS, "stk_dsd: negative size");
+    if (blocking > 0 && (m % blocking || k % blocking))
+      return fail(STK_ERR_DIMS, "incompatible dimensions: sparse [%lld, %lld] x dense [%lld, %lld] with blocking %d", (long long)m, (long long)k,
+                  (long long)k, (long long)n, blocking);
+    const bool ta = transpose_a != 0;
+    if (ta && nnz > 0 && !block_offsets_t) return fail(STK_ERR_DIMS, "stk_dsd: missing metadata pointer");
+    return walk_f32(true, "stk_dsd", blocking > 0 ? m / blocking : 0, n, data, ta ? offsets_t : offsets, ta ? column_indices_t : column_indices,
+                    ta ? block_offsets_t : nullptr, !ta, rhs, rhs_stride_n, rhs_stride_k, out, out_stride_m, nnz, blocking, index_dtype,
+                    static_cast<hipStream_t>(stream));
+  }
   DsdProblem problem;
   const int rc = dsd_problem("stk_dsd", m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, transpose_a, rhs,
                              rhs_stride_k, rhs_stride_n, out, out_stride_m, nnz, blocking, dtype, index_dtype, plan, &problem);

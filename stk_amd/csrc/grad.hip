@@ -144,6 +144,14 @@ extern "C" int stk_dsd_dds(int64_t m, int64_t k,
                            int64_t m_dds, const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k, void* out_dds, int64_t out_dds_stride,
                            int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32) {
+    // float32 values have no joint launch: the two products one after the other
+    const int first = stk_dsd(m, k, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k, rhs_stride_n,
+                              out_dsd, out_dsd_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+    if (first != STK_OK) return first;
+    return stk_dds(m_dds, m, k, lhs, lhs_stride_m, lhs_stride_k, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0,
+                   out_dds, out_dds_stride, nnz, blocking, dtype, index_dtype, plan, stream);
+  }
   DsdProblem dsd;
   DdsProblem dds;
   int rc = dsd_problem("stk_dsd_dds", m, k, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k,
@@ -182,6 +190,13 @@ extern "C" int stk_dsd_dsd(int64_t m, int64_t k,
                            int64_t n_t, const void* rhs_t, int64_t rhs_t_stride_k, int64_t rhs_t_stride_n, void* out_t, int64_t out_t_stride,
                            int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32) {
+    const int first = stk_dsd(m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k, rhs_stride_n, out,
+                              out_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+    if (first != STK_OK) return first;
+    return stk_dsd(k, m, n_t, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 1, rhs_t, rhs_t_stride_k, rhs_t_stride_n,
+                   out_t, out_t_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0, stream);
+  }
   DsdProblem plain, transposed;
   int rc = dsd_problem("stk_dsd_dsd", m, k, n, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t, 0, rhs, rhs_stride_k,
                        rhs_stride_n, out, out_stride, nnz, blocking, dtype, index_dtype, plan, &plain);
@@ -221,6 +236,14 @@ extern "C" int stk_sdd_dsd(int64_t m, int64_t n,
                            void* out_dsd, int64_t out_dsd_stride,
                            int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32) {
+    const int first = stk_sdd(lhs, lhs_stride_m, lhs_stride_k, rhs_sdd, rhs_sdd_stride_k, rhs_sdd_stride_n, m, k_sdd, n, out_sdd, offsets, row_indices,
+                              column_indices, block_offsets_t, nnz, blocking, dtype, index_dtype, plan, stream);
+    if (first != STK_OK) return first;
+    return stk_dsd(transpose_a ? n : m, transpose_a ? m : n, n_dsd, data, offsets, column_indices, offsets_t, column_indices_t, block_offsets_t,
+                   transpose_a, rhs_dsd, rhs_dsd_stride_k, rhs_dsd_stride_n, out_dsd, out_dsd_stride, nnz, blocking, dtype, index_dtype, plan, nullptr, 0,
+                   stream);
+  }
   SddProblem sdd;
   DsdProblem dsd;
   int rc = sdd_problem("stk_sdd_dsd", lhs, lhs_stride_m, lhs_stride_k, rhs_sdd, rhs_sdd_stride_k, rhs_sdd_stride_n, m, k_sdd, n, out_sdd, offsets,

@@ -246,6 +246,9 @@ extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_
                              int blocking, int dtype, int index_dtype, const uint8_t* plan,
                              int activation, const void* multiplier, stk_stream_t stream) {
   using namespace stk;
+  if (dtype == STK_F32)
+    return sdd_f32(lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, row_indices, column_indices, nnz, blocking,
+                   index_dtype, activation, multiplier, static_cast<hipStream_t>(stream));
   SddProblem problem;
   const int rc = sdd_problem("stk_sdd", lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, offsets, row_indices,
                              column_indices, block_order, nnz, blocking, dtype, index_dtype, plan, activation, multiplier, &problem);

@@ -7,7 +7,9 @@ import torch
 from oracle import stk_oracle as O
 
 # north-star tolerances against the fp32 oracle
-TOL = {torch.bfloat16: dict(rtol=1e-2, atol=1e-2), torch.float16: dict(rtol=1e-2, atol=5e-3)}
+TOL = {torch.bfloat16: dict(rtol=1e-2, atol=1e-2), torch.float16: dict(rtol=1e-2, atol=5e-3),
+       # float32 values (not part of the north-star statement): sums of up to 2048 fp32 products, two summation orders
+       torch.float32: dict(rtol=1e-4, atol=1e-5)}
 
 
 # Scale-free bounds beside them.  The absolute tolerances above exceed the size of the outputs when the
@@ -16,8 +18,8 @@ TOL = {torch.bfloat16: dict(rtol=1e-2, atol=1e-2), torch.float16: dict(rtol=1e-2
 # (bfloat16) or 2^-11 (float16) of its own size:
 #   max |got - want|  <=  MAX_REL * max |want|       (2x / 4x half an ulp of the largest element)
 #   ||got - want||_F  <=  RMS_REL * ||want||_F       (rounding noise is about 0.4 x 2^-8 resp. 2^-11 of the norm)
-MAX_REL = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -9}
-RMS_REL = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}
+MAX_REL = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -9, torch.float32: 2.0 ** -16}
+RMS_REL = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -18}
 
 
 def stable_seed(*args):

@@ -32,6 +32,9 @@ _SMALL = ((128, 64, 192, 0.0), (256, 192, 320, 0.5), (512, 256, 128, 0.8), (64, 
 
 _GRID = [(*s, *t, 128, d) for s, t, d in itertools.product(_SIZES, _TRANSPOSE, _DTYPES)]
 _GRID += [(*s, *t, 64, d) for s, t, d in itertools.product(_SMALL, _TRANSPOSE, _DTYPES)]
+# float32 values, which the reference's launchers pass on like any other dtype (stk/backend/triton_kernels.py:250, 306, 358)
+_GRID += [(*s, *t, 128, torch.float32) for s, t in itertools.product(_SIZES, _TRANSPOSE)]
+_GRID += [(*s, *t, 64, torch.float32) for s, t in itertools.product(_SMALL, _TRANSPOSE)]
 
 
 def _seed(*args):
@@ -911,14 +914,13 @@ def test_dmoe_config5_extreme_skew_full_size():
     _check_dmoe_products_full_size(top[:, None], 1024, 4096, 64, torch.float16, 6)
 
 
-@pytest.mark.parametrize("dtype", _DTYPES)
+@pytest.mark.parametrize("dtype", _DTYPES + (torch.float32,))
 def test_config1_seed0_mask_all_products(dtype):
     """BASELINE configuration 1 on the HIP path: stk.random.mask(1024, 1024, 0.5, 128) from numpy seed 0 (the
     known-answer topology of tests/golden/config1_topology.json), dense operands 1024 x 1024 ~ N(0, 1) from torch
-    seed 0 rounded to the 16-bit type the kernels compute in, sdd / dsd / dds in all four transpose variants
-    against the oracle.  (The reference runs this configuration in fp32 on the host; the products here take
-    float16 / bfloat16 device tensors only.)  With N(0, 1) operands the sums are ~32, far above the absolute
-    tolerance, so the comparison is a relative one."""
+    seed 0 - in fp32 as the configuration states, and rounded to the two 16-bit types - sdd / dsd / dds in all four
+    transpose variants against the oracle.  (The configuration on host tensors: tests/test_host_products.py.)  With
+    N(0, 1) operands the sums are ~32, far above the absolute tolerance, so the comparison is a relative one."""
     import json
     import os
     np.random.seed(0)
