@@ -19,10 +19,13 @@ launches (`per_op_ms`, `roofline`), then each product K times back to back betwe
 
 The JSON line also carries
   dense      same-problem dense bf16 GEMMs (torch.bmm over experts with the same
-             FLOPs and weight bytes) timed in the same run, and our fraction of them
+             FLOPs and weight bytes) timed in the same run, and our fraction of them; the same
+             batched products at 256 and 384 rows per expert (`whole_tiles`) and the single
+             GEMM of equal FLOPs (`frac_of_single_gemm`) beside them
   roofline   algorithmic bytes (or FLOPs) of the slowest of the three kernels over
              its mean duration from HIP events on the launch stream; `traffic` is read
-             from the rocprofv3 counter summary under profiles/ (its source is named)
+             from the rocprofv3 counter summary under profiles/ (its source and commit are
+             named; null with `traffic_stale` when the kernel sources have changed since)
   routing    the token routing on either side of the products on the same workload
              (sort into padded expert bins, gather, scatter), timed outside the step
   other_configs  per-product times on the other configurations of BASELINE.json with their
@@ -125,6 +128,18 @@ def dense_comparators(rows, dev, steps, warmup):
     wa = (torch.randn(HIDDEN, FFN, device=dev) * 0.02).bfloat16()
     ms = time_events(lambda: torch.mm(xa, wa), steps, warmup)
     out["single_gemm_tflops"] = flops / (ms * 1e-3) / 1e12
+    del xe, he, xa
+    # the same batched products with 256 and 384 token rows per expert: whole macro-tiles of the library's kernels
+    # (the mean of the routed counts, 314 rows here, is a ragged size for them), so that the comparator is not one
+    # the library happens to be slow at
+    out["whole_tiles"] = {}
+    for t in (256, 384):
+        xt = (torch.randn(EXPERTS, t, HIDDEN, device=dev) * 0.02).bfloat16()
+        ht = torch.bmm(xt, w1)
+        f = 2.0 * EXPERTS * t * HIDDEN * FFN
+        fns = {"sdd": lambda: torch.bmm(xt, w1), "dsd": lambda: torch.bmm(ht, w2), "dds": lambda: torch.bmm(xt.transpose(1, 2), ht)}
+        out["whole_tiles"][str(t)] = {k + "_like_tflops": f / (time_events(fn, steps, warmup) * 1e-3) / 1e12 for k, fn in fns.items()}
+        del xt, ht
     return out
 
 
@@ -427,22 +442,53 @@ def other_config(name, dev, steps, warmup):
 
 # HBM bytes per launch on this workload come from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, scaled by what the
 # same counters read for a plain copy of known size); the tracked summary of that run is read here, so that the
-# figure in the JSON line is the one in the repository and names its source.
+# figure in the JSON line is the one in the repository and names its source.  The summary records the digest of the
+# kernel sources it was taken with (`kernel_sources_sha256:`, printed by `bench.py --kernel-sources-digest`) and the
+# commit; when the sources in the tree differ, the counters describe other kernels than the ones just timed and the
+# line carries no traffic at all rather than a stale one.
 HBM_COUNTER_SUMMARY = os.path.join("profiles", "bench_dmoe_fwd_hbm_counters.txt")
 
 
-def measured_hbm_traffic(kernel):
-    """(bytes per launch, source) for `kernel` from the 'total MB' column of the counter summary, or (None, reason)."""
-    path = os.path.join(ROOT, HBM_COUNTER_SUMMARY)
+def kernel_sources_digest(root=ROOT):
+    """sha256 over the device sources of the library (stk_amd/csrc/*.hip and *.h, names and contents, sorted)."""
+    import hashlib
+    csrc = os.path.join(root, "stk_amd", "csrc")
+    digest = hashlib.sha256()
+    for name in sorted(n for n in os.listdir(csrc) if n.endswith((".hip", ".h"))):
+        digest.update(name.encode() + b"\0")
+        with open(os.path.join(csrc, name), "rb") as f:
+            digest.update(f.read())
+    return digest.hexdigest()
+
+
+def counter_summary(path=None):
+    """{'kernels': {name: bytes per launch}, 'sha256': ..., 'commit': ..., 'stale': bool, 'problem': text or None}."""
+    path = path or os.path.join(ROOT, HBM_COUNTER_SUMMARY)
+    info = {"kernels": {}, "sha256": None, "commit": None, "stale": True, "problem": None}
     try:
         with open(path) as f:
             for line in f:
                 parts = line.split()
-                if len(parts) >= 8 and parts[0] == kernel:
-                    return float(parts[5]) * 1e6, HBM_COUNTER_SUMMARY
+                if len(parts) >= 8 and parts[0].endswith("_kernel") and parts[0] not in info["kernels"]:
+                    try:
+                        info["kernels"][parts[0]] = float(parts[5]) * 1e6      # the 'total MB' column
+                    except ValueError:
+                        pass
+                elif len(parts) == 2 and parts[0] == "kernel_sources_sha256:":
+                    info["sha256"] = parts[1]
+                elif len(parts) == 2 and parts[0] == "commit:":
+                    info["commit"] = parts[1]
     except OSError as err:
-        return None, f"{HBM_COUNTER_SUMMARY}: {err.strerror}"
-    return None, f"{HBM_COUNTER_SUMMARY}: no line for {kernel}"
+        info["problem"] = f"{HBM_COUNTER_SUMMARY}: {err.strerror}"
+        return info
+    if info["sha256"] is None:
+        info["problem"] = f"{HBM_COUNTER_SUMMARY} does not say which kernel sources it was taken with"
+    elif info["sha256"] != kernel_sources_digest():
+        info["problem"] = (f"{HBM_COUNTER_SUMMARY} was taken at commit {info['commit']} with other kernel sources than the tree holds: "
+                           "its traffic figures are not reported (collect the counters again)")
+    else:
+        info["stale"] = False
+    return info
 
 
 def main():
@@ -458,9 +504,14 @@ def main():
                     help="also run one plain 1 GiB -> 1 GiB elementwise kernel (torch.neg), the known-size reference for the HBM counters")
     ap.add_argument("--gradient-pair-only", action="store_true",
                     help="run only the gradient pairs of sdd and of dsd, each as one launch and as two (for the counter profiles)")
+    ap.add_argument("--kernel-sources-digest", action="store_true",
+                    help="print the digest of the kernel sources that a counter summary under profiles/ records, and exit")
     ap.add_argument("--configs", default="2,4,5,5skew",
                     help="comma-separated other configurations of BASELINE.json to time as well (2, 4, 5, 5skew); 'none' leaves them out")
     args = ap.parse_args()
+    if args.kernel_sources_digest:
+        print(kernel_sources_digest())
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the block-sparse products have no multi-GPU path in this build (--gpus must be 1)")
     extra = [c for c in args.configs.split(",") if c and c != "none"]
@@ -600,12 +651,21 @@ def main():
         achieved = per_op_tflops[dominant]
         roof = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS}
     kernel_names = {"sdd": "sdd_fused_kernel", "dsd": "dsd_sliced_kernel", "dds": "dds_fused_kernel"}
-    traffic, traffic_source = measured_hbm_traffic(kernel_names[dominant])
-    roof.update({"traffic": traffic, "traffic_source": traffic_source, "kernel": kernel_names[dominant], "avg_launch_ms": per_op_ms[dominant],
+    counters = counter_summary()
+    if counters["problem"]:
+        print("bench.py: " + counters["problem"], file=sys.stderr)
+
+    def traffic_of(n):
+        return None if counters["stale"] else counters["kernels"].get(kernel_names[n])
+
+    roof.update({"traffic": traffic_of(dominant), "traffic_source": HBM_COUNTER_SUMMARY, "traffic_commit": counters["commit"],
+                 "traffic_stale": counters["stale"], "kernel": kernel_names[dominant], "avg_launch_ms": per_op_ms[dominant],
                  "algorithmic_bytes": bytes_op[dominant], "flops": flops_op,
                  "per_kernel": {kernel_names[n]: {"avg_launch_ms": per_op_ms[n], "algorithmic_bytes": bytes_op[n],
                                                   "frac_of_hbm_peak": bytes_op[n] / (per_op_ms[n] * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                                  "traffic": measured_hbm_traffic(kernel_names[n])[0]} for n in names}})
+                                                  "traffic": traffic_of(n)} for n in names}})
+    if counters["problem"]:
+        roof["traffic_note"] = counters["problem"]
 
     result = {
         "metric": "nonzero-block TFLOP/s for SDD/DSD/DDS; % of dense bf16 GEMM at dMoE shape",
@@ -625,6 +685,9 @@ def main():
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "dense": dense, "frac_of_dense_per_op": frac_dense, "frac_of_dense_per_op_back_to_back": frac_dense_b2b,
         "frac_of_dense_step": value / dense_step_tflops,
+        # against the one plain GEMM of the same FLOPs, which reads 1/64 of the weights (an upper bound, not the same problem)
+        "frac_of_single_gemm": {n: per_op_tflops[n] / dense["single_gemm_tflops"] for n in names},
+        "frac_of_dense_whole_tiles": {t: {n: per_op_tflops[n] / d[n + "_like_tflops"] for n in names} for t, d in dense["whole_tiles"].items()},
         "roofline": roof,
         "routing": routing,
         "sdd_gradient_pair": gradient_pair,

@@ -51,16 +51,16 @@ def assert_close(got, want, dtype, what=""):
                              f"first at {tuple(idx)}: got {got[tuple(idx)]} want {want[tuple(idx)]}")
 
 
-def assert_close_scaled(got, want, dtype, what=""):
-    """The north-star tolerance and the two scale-free bounds, for tensors on any device (computed there,
-    so that full-size results need not travel to the host).  `want` is the fp32 reference."""
+def assert_close_scaled(got, want, dtype, what="", tol=None):
+    """The north-star tolerance (or `tol`) and the two scale-free bounds, for tensors on any device (computed
+    there, so that full-size results need not travel to the host).  `want` is the fp32 reference."""
     got = got.detach().float() if isinstance(got, torch.Tensor) else torch.as_tensor(np.asarray(got, dtype=np.float32))
     want = want.detach().float() if isinstance(want, torch.Tensor) else torch.as_tensor(np.asarray(want, dtype=np.float32))
     want = want.to(got.device)
     assert got.shape == want.shape, (what, tuple(got.shape), tuple(want.shape))
     if got.numel() == 0:
         return
-    tol = TOL[dtype]
+    tol = tol or TOL[dtype]
     bad = ~torch.isclose(got, want, **tol)
     if bool(bad.any()):
         idx = tuple(int(i) for i in bad.nonzero()[0])

@@ -205,6 +205,28 @@ def test_bench_rejects_what_it_does_not_measure():
         assert text in run.stderr, run.stderr
 
 
+def test_bench_reports_no_traffic_from_counters_taken_with_other_kernel_sources(tmp_path):
+    # roofline.traffic comes from a tracked counter summary; it is only reported while the kernel sources are the ones
+    # the counters were taken with
+    import bench
+    digest = bench.kernel_sources_digest()
+    assert len(digest) == 64 and digest == bench.kernel_sources_digest()
+    row = "  dds_fused_kernel       100779.6     524670.4     206.4      537.3      743.7            742.7    1.00\n"
+    fresh = tmp_path / "fresh.txt"
+    fresh.write_text("commit: abc1234\nkernel_sources_sha256: " + digest + "\n" + row)
+    info = bench.counter_summary(str(fresh))
+    assert not info["stale"] and info["problem"] is None and info["commit"] == "abc1234"
+    assert info["kernels"]["dds_fused_kernel"] == pytest.approx(743.7e6)
+    stale = tmp_path / "stale.txt"
+    stale.write_text("commit: abc1234\nkernel_sources_sha256: " + "0" * 64 + "\n" + row)
+    info = bench.counter_summary(str(stale))
+    assert info["stale"] and "other kernel sources" in info["problem"]
+    unmarked = tmp_path / "unmarked.txt"
+    unmarked.write_text(row)
+    assert bench.counter_summary(str(unmarked))["stale"]
+    assert bench.counter_summary(str(tmp_path / "missing.txt"))["stale"]
+
+
 def test_dsd_workspace_choice():
     # captured launches never touch the device's shared workspace; eager launches share it and serialise across streams
     from stk_amd.backend.hip_kernels import _workspace_choice
