@@ -78,31 +78,86 @@ __global__ __launch_bounds__(512, 2) void dds_fused64_kernel(DdsArgs g, PlanList
 
 // 128-blocks, eight wavefronts: 256x256 tiles over the pairs of identical block columns, then
 // 256x128 tiles over the lone ones, taken from the lists of the plan (covered columns get no
-// workgroup; the grid is an upper bound and the surplus leaves at once).  Without a plan every
-// column is a lone column.
+// tile).  Without a plan every column is a lone column.
+//
+// One workgroup of this kernel fills a compute unit (its ring takes most of the LDS), so the grid is one workgroup
+// per compute unit and every workgroup walks the tiles with the stride of the grid - the order in which the hardware
+// would hand them out one launch at a time, without the launch (0.75 us per tile, measured with an empty kernel on
+// the same grid) and without the three dependent loads of a tile's walk (list entry, offsets, entries: 1.1 us) in
+// front of its first transfer: the walk of the next tile is looked up through the scalar unit while the first
+// transfers of the current one are in flight.
+// The id of the tile that a workgroup takes in its round `round` of a launch of one workgroup per compute unit: the
+// tiles of a round are consecutive ids, and a workgroup keeps its compute die (id mod 8, the die its own id lies on),
+// but odd rounds hand the tiles of a die out in reverse.  A list sorted by length then gives every workgroup a long
+// tile of one round and a short one of the next, as the hardware's own hand-out to whoever is free first would.
+__device__ __forceinline__ int round_tile(int round) {
+  const int slots = gridDim.x >> 3, die = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  if ((gridDim.x & 7) || !(round & 1)) return round * gridDim.x + blockIdx.x;
+  return round * gridDim.x + (slots - 1 - slot) * 8 + die;
+}
+
+// The tiles [first, first + count) of the launch, all of LINES block columns, that this workgroup takes (round_tile);
+// locate(id) gives a tile's first block column and first output row.  `round` counts on from the call before.
+template <class Cfg, bool TRANS_B, int LINES, class Locate>
+__device__ __forceinline__ void dds_walk_tiles(const DdsArgs& g, int first, int count, Locate&& locate, char* smem, int& round, bool& used_lds) {
+  int id = round_tile(round);
+  while (id < first) id = round_tile(++round);
+  if (id >= first + count) return;
+  int line, m0;
+  locate(id, line, m0);
+  DdsWalk<LINES> walk;
+  if (!dds_walk_scalar<LINES, TRANS_B>(g, line, LINES, walk)) walk = dds_walk<LINES, TRANS_B>(g, line, LINES);
+  for (;;) {
+    if (used_lds) __syncthreads();  // the staging area of the last tile's stores is the first ring stage of this one
+    used_lds = true;
+    const int next_id = round_tile(++round);
+    const bool more = next_id < first + count;
+    int next_line = line, next_m0 = m0;
+    DdsWalk<LINES> next_walk = walk;
+    bool have_next = false;
+    auto look_ahead = [&] {
+      if (more) {
+        locate(next_id, next_line, next_m0);
+        have_next = dds_walk_scalar<LINES, TRANS_B>(g, next_line, LINES, next_walk);
+      }
+    };
+    if (walk.nseg <= 0) look_ahead();  // (a column without blocks has no main loop to hide it behind)
+    dds_tile_of<Cfg, 128, TRANS_B, true, LINES>(g, walk, m0, smem, LINES, look_ahead);
+    if (!more) return;
+    id = next_id;
+    line = next_line;
+    m0 = next_m0;
+    if (have_next) walk = next_walk;
+    else walk = dds_walk<LINES, TRANS_B>(g, line, LINES);
+  }
+}
+
 template <class Fused, class Single, bool TRANS_B>
 __global__ __launch_bounds__(512, 2) void dds_fused_kernel(DdsArgs g, PlanLists plan) {
   extern __shared__ __align__(16) char smem[];
   static_assert(Fused::TM == Single::TM, "same row tiling");
   const int ntm = g.m / Fused::TM;
-  int bid = blockIdx.x;
+  bool used_lds = false;
+  int round = 0;
   if (!plan.counts) {
-    const int item = xcd_grouped(bid, g.block_cols * ntm);
-    dds_tile<Single, 128, TRANS_B, true, 1>(g, item / ntm, (item % ntm) * Single::TM, smem);
+    const int total = g.block_cols * ntm;
+    dds_walk_tiles<Single, TRANS_B, 1>(g, 0, total, [&](int id, int& line, int& m0) {
+      const int item = xcd_grouped(id, total);
+      line = item / ntm, m0 = (item % ntm) * Single::TM;
+    }, smem, round, used_lds);
     return;
   }
   const int pair_tiles = const_ints(plan.counts)[kPairs] * ntm, single_tiles = const_ints(plan.counts)[kSingles] * ntm;
-  if (bid < pair_tiles) {
-    const int item = xcd_item(bid, pair_tiles, ntm, plan.group(kPairs));
-    dds_tile<Fused, 128, TRANS_B, true, 2>(g, const_ints(plan.list(kPairs))[item / ntm], (item % ntm) * Fused::TM, smem);
-    return;
-  }
-  bid -= pair_tiles;
-  if (bid < single_tiles) {
-    // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
-    const int item = xcd_lines(bid, single_tiles, ntm, (plan.stripe_from(false) + 1) >> 1);
-    dds_tile<Single, 128, TRANS_B, true, 1>(g, const_ints(plan.list(kSingles))[item / ntm], (item % ntm) * Single::TM, smem);
-  }
+  dds_walk_tiles<Fused, TRANS_B, 2>(g, 0, pair_tiles, [&](int id, int& line, int& m0) {
+    const int item = xcd_item(id, pair_tiles, ntm, plan.group(kPairs));
+    line = const_ints(plan.list(kPairs))[item / ntm], m0 = (item % ntm) * Fused::TM;
+  }, smem, round, used_lds);
+  // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
+  const int stripe_from = (plan.stripe_from(false) + 1) >> 1;
+  dds_walk_tiles<Single, TRANS_B, 1>(g, pair_tiles, single_tiles, [&](int id, int& line, int& m0) {
+    const int item = xcd_lines(id - pair_tiles, id, single_tiles, ntm, stripe_from);
+    line = const_ints(plan.list(kSingles))[item / ntm], m0 = (item % ntm) * Single::TM;
+  }, smem, round, used_lds);
 }
 
 template <class Cfg, int BLK, bool TRANS_B, bool FULL>
@@ -130,7 +185,9 @@ static void launch_dds(const DdsArgs& g, const PlanLists& plan, hipStream_t stre
       constexpr int lds = Fused::kSmemBytes > Single::kSmemBytes ? Fused::kSmemBytes : Single::kSmemBytes;
       static const int once = (set_lds_limit(&dds_fused_kernel<Fused, Single, TRANS_B>, lds), 0);
       (void)once;
-      hipLaunchKernelGGL((dds_fused_kernel<Fused, Single, TRANS_B>), dim3(g.block_cols * (g.m / Fused::TM)), dim3(512), lds, stream, g, plan);
+      // one workgroup per compute unit; the tiles are at most one per block column and row tile
+      const int units = compute_units(), tiles = g.block_cols * (g.m / Fused::TM);
+      hipLaunchKernelGGL((dds_fused_kernel<Fused, Single, TRANS_B>), dim3(units > 0 && units < tiles ? units : tiles), dim3(512), lds, stream, g, plan);
     } else if (g.m % Narrow::TM == 0 && plan.counts) {
       static const int once = (set_lds_limit(&dds_lines_kernel<Narrow, BLK, TRANS_B>, Narrow::kSmemBytes), 0);
       (void)once;
@@ -212,6 +269,7 @@ int stk::dds_problem(const char* who, int64_t m, int64_t k, int64_t n,
   p->ak = ak;
   p->tb = tb;
   g.small = nnz * (m / 128) < kSmallWorkPerUnit * compute_units();
+  g.scalar_walk = ((reinterpret_cast<uintptr_t>(g.walk_columns) | reinterpret_cast<uintptr_t>(g.walk_blocks)) & 3u) == 0;
   if (!g.walk_offsets || (nnz > 0 && (!g.walk_columns || (!tb && !g.walk_blocks) || !data))) return fail(STK_ERR_DIMS, "%s: missing metadata pointer", who);
   // lists of the walked lines: block columns of the stored matrix [k, n], or block rows of the stored [n, k]
   p->lists = PlanLists{nullptr, nullptr, 0};

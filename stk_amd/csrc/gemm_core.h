@@ -433,9 +433,11 @@ __device__ __forceinline__ void static_for(Fn&& fn) {
 
 // Full tiles: direct-to-LDS pipeline.  tile_fn(t) gives the operand origins of
 // K-tile t; it is called exactly once per t, in increasing order.
-template <class Cfg, class TileFn>
+// after_prologue() runs once, behind the transfers of the first STAGES - 1 K-tiles and in front of the first wait: work
+// that does not depend on the tile (the caller's look-ahead) sits there in the shadow of the first transfers' latency.
+template <class Cfg, class TileFn, class Hook>
 __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
-                                             int64_t lda, int64_t ldb, char* smem) {
+                                             int64_t lda, int64_t ldb, char* smem, Hook&& after_prologue) {
   using OpA = typename Cfg::OpA;
   using OpB = typename Cfg::OpB;
   constexpr int S = Cfg::STAGES;
@@ -481,6 +483,7 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
 #pragma unroll
   for (int s = 0; s < S - 1; s++)
     if (s < ntiles) issue(s);
+  after_prologue();
 
   if constexpr (Cfg::WK == 1 && S >= 3) {
     // Software pipeline over the MFMA k-steps: the fragments of the next k-step are read
@@ -591,6 +594,12 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
   }
   __syncthreads();  // operand reads done before the epilogue reuses LDS
 }
+template <class Cfg, class TileFn>
+__device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
+                                             int64_t lda, int64_t ldb, char* smem) {
+  mainloop_dma<Cfg>(acc, ntiles, tile_fn, lda, ldb, smem, [] {});
+}
+
 // Ragged tiles: predicated register staging, two LDS stages.
 template <class Cfg, class TileFn>
 __device__ __forceinline__ void mainloop_reg(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
@@ -650,9 +659,12 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
                                          int m_valid, int n_valid, char* smem, int64_t quadrant_stride = 64,
                                          int activation = kNoActivation, const elem_t* mul = nullptr,
                                          int row_base = 0, int64_t row_jump = 0) {
-  const int tid = threadIdx.x;
+  // (the thread's id through an opaque statement: in a workgroup that loops over tiles the store addresses below would
+  // otherwise be computed once in front of the loop and held in registers through every K loop)
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   if constexpr (Cfg::WK == 1) {
     char* s = smem + wave * 8192;  // [64 m][64 n] 16-bit, rows of 128 bytes, 8-byte units swizzled by the row
 #pragma unroll
@@ -800,18 +812,20 @@ __device__ __forceinline__ int xcd_item(int bid, int n, int per, int entries) {
   return base + (r & 7) * group + (r >> 3);
 }
 // Tiles of a list of single lines, `per` tiles of the dense operand for each line (item = line index * per + dense
-// tile); bid counts from the list's first tile.  From `stripe_from` dense tiles on (0: never; the plan's hint) and
+// tile); bid counts from the list's first tile and id is the workgroup's id in the whole launch (for a workgroup
+// that walks several tiles: the id a launch of one workgroup per tile would give this tile).  From `stripe_from` dense tiles on (0: never; the plan's hint) and
 // when they divide by the eight dies, die d takes the dense tiles [d per / 8, (d + 1) per / 8) of every line, in the
 // order of the lines: it then fetches its stripe of the dense operand once, whichever lines need it.  Otherwise
 // groups of neighbouring items.
-__device__ __forceinline__ int xcd_lines(int bid, int n, int per, int stripe_from) {
+__device__ __forceinline__ int xcd_lines(int bid, int id, int n, int per, int stripe_from) {
   if (stripe_from == 0 || per < stripe_from || (per & 7)) return xcd_grouped(bid, n);
   // the workgroup's die, and how many of the list's tiles the die has taken before this one
-  const int id = blockIdx.x, first = id - bid, die = id & 7;
+  const int first = id - bid, die = id & 7;
   const int local = (id >> 3) - ((first + 7 - die) >> 3);
   const int share = per >> 3;
   return (local / share) * per + die * share + local % share;
 }
+__device__ __forceinline__ int xcd_lines(int bid, int n, int per, int stripe_from) { return xcd_lines(bid, blockIdx.x, n, per, stripe_from); }
 // The tiles of stk_sdd: groups of eight.  Measured against eight contiguous shares of the tile list: the same or up
 // to 6 % faster (equal shares of a list are unequal shares of the work when the experts differ in size).
 #ifndef STK_XCD_SDD_GROUP
