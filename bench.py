@@ -280,6 +280,52 @@ def routing_times(dev, steps, warmup, seed=0):
         out[name + "_frac_of_hbm_peak"] = out[name + "_gbs"] / PEAK_HBM_GBS
         out[name + "_op_ms"] = time_events(op, steps, warmup)
     assert torch.equal(gathered, padded) and torch.equal(scattered, x)
+    out["routed_forward"] = routed_forward_times(x, r, warmup)
+    return out
+
+
+def routed_forward_times(x, r, warmup, calls=20):
+    """The forward pass of the routed layer on the benchmark workload, tokens in and tokens out, as the four launches
+    gather -> sdd(gelu) -> dsd -> scatter and as the two launches that read and write the token rows in place
+    (stk_sdd_gather, stk_dsd_scatter); outputs allocated once, `calls` passes back to back between one pair of events."""
+    import stk_amd as stk
+    from stk_amd.backend import hip_kernels
+    dev, rows = x.device, r.row_slots.numel()
+    topo = stk.ops.dmoe_topology(r.padded_bins, BLOCK, rows // BLOCK, FFN // BLOCK, dtype=torch.bfloat16)
+    w1 = (torch.randn(HIDDEN, EXPERTS * FFN, device=dev) * 0.02).bfloat16()
+    w2 = (torch.randn(EXPERTS * FFN, HIDDEN, device=dev) * 0.02).bfloat16()
+    meta = (topo.offsets, topo.row_indices, topo.column_indices)
+    walk = (topo.offsets, topo.row_indices, topo.column_indices, topo.offsets_t, topo.column_indices_t, topo.block_offsets_t)
+    h = torch.empty_like(topo.data)
+    padded_y, y4, y2 = torch.empty(rows, HIDDEN, dtype=x.dtype, device=dev), None, torch.empty_like(x)
+
+    def four():
+        nonlocal y4
+        padded = hip_kernels.padded_gather(x, r.row_slots, 1)
+        hip_kernels.sdd_fused(padded, w1, topo.size(), h, *meta, "gelu_tanh")
+        hip_kernels.dsd(topo.size(), h, *walk, False, w2, padded_y)
+        y4 = hip_kernels.padded_scatter(padded_y, r.slot_rows, 1)
+
+    def two():
+        assert hip_kernels.sdd_gather(x, r.row_slots, 1, w1, topo.size(), h, *meta, "gelu_tanh")
+        assert hip_kernels.dsd_scatter(topo.size(), h, topo.offsets, topo.column_indices, topo.offsets_t, topo.column_indices_t, w2,
+                                       r.row_slots, None, y2)
+
+    def back_to_back(fn):
+        for _ in range(warmup):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(calls):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / calls
+
+    out = {"four_launches_ms": back_to_back(four), "two_launches_ms": back_to_back(two)}
+    out["saved_us"] = (out["four_launches_ms"] - out["two_launches_ms"]) * 1e3
+    out["bit_identical"] = bool(torch.equal(y4, y2))
     return out
 
 

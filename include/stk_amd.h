@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 14
+#define STK_AMD_ABI_VERSION 15
 
 /* status codes */
 #define STK_OK 0
@@ -461,6 +461,41 @@ int stk_padded_scatter_weight_gradient(const void* x, int64_t padded_rows, int64
                                        const void* grad, int64_t grad_stride,
                                        const int32_t* slot_rows, int top_k, int64_t tokens,
                                        float* out, int dtype, stk_stream_t stream);
+
+/*
+ * stk_padded_gather (weights NULL) and stk_sdd_fused in one launch: the sampled product of the padded layout's rows
+ * with rhs, read straight from the token rows, so that the padded copy of the tokens is neither written nor read.
+ *   out (nnz blocks) = act(lhs [m, k] * rhs [k, n]) on the topology,  lhs[r] = tokens[row_slots[r] / top_k],
+ * a row of zeros where row_slots[r] is not in [0, num_tokens * top_k).  tokens is [num_tokens, k], row-major with
+ * token_stride elements between rows; row_slots has m entries (stk_route writes it).  The other arguments are those of
+ * stk_sdd_fused (no block_order, no multiplier; activation one of STK_ACT_NONE .. STK_ACT_SILU, which map the zero
+ * rows to zeros).  Bit-identical to the two calls it replaces.  128-blocks only, and the token rows must span less
+ * than 4 GiB; STK_ERR_UNSUPPORTED otherwise (callers then make the two calls).  No counterpart in the reference,
+ * whose callers gather with their own kernels (see stk_route) in front of sdd, stk/backend/sputnik.py:206-237.
+ */
+int stk_sdd_gather(const void* tokens, int64_t num_tokens, int64_t token_stride, const int32_t* row_slots, int top_k,
+                   const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n, int64_t m, int64_t k, int64_t n,
+                   void* out, const int32_t* offsets, const void* row_indices, const void* column_indices, int64_t nnz,
+                   int blocking, int dtype, int index_dtype, const uint8_t* plan, int activation, stk_stream_t stream);
+
+/*
+ * stk_dsd (sparse operand not transposed) and stk_padded_scatter for top_k = 1 in one launch: the rows of
+ * S [m, k] * rhs [k, n] go straight to the token rows they belong to, so that the padded result is neither written
+ * nor read.
+ *   out[row_slots[r]] = (weights[row_slots[r]] *) (S * rhs)[r]   for every r with row_slots[r] in [0, num_tokens)
+ * The sums are rounded to dtype, then multiplied by the fp32 weight and rounded again (weights NULL: not at all),
+ * which is what the two calls do; the results are theirs bit for bit.  Rows of `out` that no r names are not
+ * written (stk_route with top_k = 1 names every token).  out is [num_tokens, n] with out_stride_m elements between
+ * rows.  The other arguments are those of stk_dsd, workspace included.  128-blocks, n a multiple of 256 and a launch
+ * that stk_dsd would run on its eight-wavefront tiles only; STK_ERR_UNSUPPORTED otherwise (callers then make the two
+ * calls).  No counterpart in the reference (see stk_route); replaces its dsd, stk/backend/sputnik.py:51-120, for
+ * this use.
+ */
+int stk_dsd_scatter(int64_t m, int64_t k, int64_t n, const void* data, const int32_t* offsets, const void* column_indices,
+                    const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                    const int32_t* row_slots, const float* weights, int64_t num_tokens, void* out, int64_t out_stride_m,
+                    int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                    void* workspace, int64_t workspace_bytes, stk_stream_t stream);
 
 #ifdef __cplusplus
 }

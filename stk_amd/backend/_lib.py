@@ -11,7 +11,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
 STK_F16, STK_BF16, STK_F32 = 0, 1, 2
 STK_I16, STK_I32 = 0, 1
@@ -55,6 +55,8 @@ SIGNATURES = {
     "stk_padded_gather": (_int, [_p, _i64, _i64, _i64, _p, _p, _int, _i64, _p, _i64, _int, _p]),
     "stk_padded_scatter": (_int, [_p, _i64, _i64, _i64, _p, _p, _int, _i64, _p, _i64, _int, _p]),
     "stk_padded_scatter_weight_gradient": (_int, [_p, _i64, _i64, _i64, _p, _i64, _p, _int, _i64, _p, _int, _p]),
+    "stk_sdd_gather": (_int, [_p, _i64, _i64, _p, _int, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _int, _p]),
+    "stk_dsd_scatter": (_int, [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _p, _i64, _p, _i64, _i64, _int, _int, _int, _p, _p, _i64, _p]),
 }
 
 _lock = threading.Lock()

@@ -700,3 +700,73 @@ def padded_scatter_weight_gradient(x, grad, slot_rows, top_k):
             x.data_ptr(), x.size(0), x.size(1), _row_stride(x), grad.data_ptr(), _row_stride(grad), slot_rows.data_ptr(), top_k,
             grad.size(0), out.data_ptr(), _value_dtype(x), _stream()))
     return out
+
+
+def sdd_gather(x, row_slots, top_k, rhs, shape, out, offsets, row_indices, column_indices, activation=None):
+    """out = act(sdd(padded_gather(x, row_slots, top_k), rhs)) on the topology without the padded copy of x
+    (stk_sdd_gather); bit-identical to padded_gather followed by sdd_fused.  False, with nothing launched, when
+    the library has no such kernel for this case (the caller then makes the two calls); True otherwise."""
+    _need_gpu(x, row_slots, rhs, out)
+    m, n = shape
+    b = _blocking(out)
+    nnz = row_indices.numel()
+    if b != 128 or activation not in ACTIVATIONS or ACTIVATIONS[activation] > ACTIVATIONS["silu"] or FUSION is False:
+        return False
+    x = _rows16(x.detach())
+    tokens, k = x.shape
+    assert k == rhs.shape[0] and n == rhs.shape[1], "incompatible dimensions"
+    assert row_slots.dtype == torch.int32 and row_slots.is_contiguous() and row_slots.numel() >= m
+    _validate_matmul_dims(m, k, n, b)
+    if tokens == 0 or tokens * _row_stride(x) * 2 >= 1 << 32:
+        return False
+    if nnz == 0:
+        return True
+    rhs = _dense_operand(rhs)
+    assert out.is_contiguous() and x.dtype == rhs.dtype == out.dtype
+    ri, ci = _index(row_indices), _index(column_indices)
+    plan = fusion_plan(offsets, column_indices, blocking=b) if offsets is not None else None
+    with _on_device(out.device):
+        status = _lib.load().stk_sdd_gather(
+            x.data_ptr(), tokens, _row_stride(x), row_slots.data_ptr(), top_k, rhs.data_ptr(), rhs.stride(0), rhs.stride(1),
+            m, k, n, out.data_ptr(), _offsets(offsets).data_ptr() if plan is not None else None, ri.data_ptr(), ci.data_ptr(), nnz,
+            b, _value_dtype(out), _INDEX_DTYPES[ri.dtype], plan.data_ptr() if plan is not None else None, ACTIVATIONS[activation], _stream())
+    if status == _lib.STK_ERR_UNSUPPORTED:
+        return False
+    _lib.check(status)
+    return True
+
+
+def dsd_scatter(shape, data, offsets, column_indices, offsets_t, column_indices_t, rhs, row_slots, weights, out):
+    """out = padded_scatter(sparse @ rhs, top_k = 1, weights) without the padded result (stk_dsd_scatter): row r of
+    the product goes to out[row_slots[r]]; bit-identical to dsd followed by padded_scatter.  False, with nothing
+    launched, when the library has no such kernel for this case (the caller then makes the two calls); True otherwise."""
+    _need_gpu(data, rhs, row_slots, out)
+    m, k = shape
+    n = rhs.shape[1]
+    b = _blocking(data)
+    assert k == rhs.shape[0], "incompatible dimensions"
+    _validate_matmul_dims(m, k, n, b)
+    tokens = out.shape[0]
+    if b != 128 or n % 256 or not FUSION or data.shape[0] == 0 or tokens == 0:
+        return False
+    rhs = _dense_operand(rhs)
+    data = data.detach()
+    assert data.is_contiguous() and out.stride(1) == 1 and out.shape[1] == n
+    assert data.dtype == rhs.dtype == out.dtype
+    assert row_slots.dtype == torch.int32 and row_slots.is_contiguous() and row_slots.numel() >= m
+    w = _weights32(weights, tokens)
+    ci = _index(column_indices)
+    plan = fusion_plan(offsets, column_indices, offsets_t, column_indices_t, blocking=b)
+    with _on_device(out.device):
+        ws = _dsd_workspace(out.device, m, n, b)
+        status = _lib.load().stk_dsd_scatter(
+            m, k, n, data.data_ptr(), _offsets(offsets).data_ptr(), ci.data_ptr(), rhs.data_ptr(), rhs.stride(0), rhs.stride(1),
+            row_slots.data_ptr(), None if w is None else w.data_ptr(), tokens, out.data_ptr(), out.stride(0),
+            data.shape[0], b, _value_dtype(out), _INDEX_DTYPES[ci.dtype], plan.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream())
+        if status == _lib.STK_ERR_UNSUPPORTED:
+            return False
+        if status != _lib.STK_OK and ws is not None:
+            release_workspaces()
+        _lib.check(status)
+    return True

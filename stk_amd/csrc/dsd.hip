@@ -83,17 +83,18 @@ __global__ __launch_bounds__(512, 2) void dsd_fused64_kernel(DsdArgs g, PlanList
 // 128-blocks, eight wavefronts.  The workgroups take their tiles from the lists of the plan (dsd_plan_tile).
 // Covered rows get no workgroup; the grid is an upper bound and the surplus leaves at once.
 // Without a plan every row is a lone row.
-template <class Fused, class Triple, class Single, bool TRANS_A>
+// SCATTER: the rows of the result are scattered (DsdArgs::row_map).
+template <class Fused, class Triple, class Single, bool TRANS_A, bool SCATTER = false>
 __global__ __launch_bounds__(512, 2) void dsd_fused_kernel(DsdArgs g, PlanLists plan) {
   extern __shared__ __align__(16) char smem[];
   int bid = blockIdx.x;
   if (!plan.counts) {
     const int ntn = g.n / Fused::TN;
     const int item = xcd_grouped(bid, g.block_rows * ntn);
-    dsd_tile<Single, 128, TRANS_A, true, 1>(g, item / ntn, (item % ntn) * Single::TN, smem);
+    dsd_tile<Single, 128, TRANS_A, true, 1, SCATTER>(g, item / ntn, (item % ntn) * Single::TN, smem);
     return;
   }
-  dsd_plan_tile<Fused, Triple, Single, TRANS_A>(g, plan, bid, smem);
+  dsd_plan_tile<Fused, Triple, Single, TRANS_A, SCATTER>(g, plan, bid, smem);
 }
 
 // ---------------------------------------------------------------------------
@@ -145,7 +146,7 @@ __device__ __forceinline__ void add_slices_in_order(f32x16_t (&acc)[Cfg::IM][Cfg
 
 // Slice `slice` of `slices` of the tile (LINES block rows from bi, columns from n0), the `ordinal`-th tile of the last
 // round; the tile owns the slots [ordinal * slices, (ordinal + 1) * slices) of the workspace.
-template <class Cfg, bool TRANS_A, int LINES>
+template <class Cfg, bool TRANS_A, int LINES, bool SCATTER = false>
 __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, int bi, int n0, int slice, int slices, int ordinal, char* smem, int* flag) {
   constexpr int kAcc = Cfg::IM * Cfg::JN;
   static_assert(kAcc * 16 * 512 <= kSlotFloats, "slot too small");
@@ -158,7 +159,7 @@ __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, i
   f32x16_t acc[Cfg::IM][Cfg::JN] = {};
   dsd_accumulate<Cfg, 128, TRANS_A, true, LINES>(acc, g, bi, n0, e0, e1, smem);
   if (slices == 1) {
-    dsd_store<Cfg, 128>(acc, g, bi, n0, smem);
+    dsd_store<Cfg, 128, SCATTER>(acc, g, bi, n0, smem);
     return;
   }
   // Partial tiles and the counter are read and written with device-scope atomic accesses only: these
@@ -218,11 +219,11 @@ __device__ __forceinline__ void dsd_slice(const DsdArgs& g, const TailArgs& t, i
       default: add_slices_in_order<Cfg, 4, 3>(acc, first); break;
     }
   }
-  dsd_store<Cfg, 128>(acc, g, bi, n0, smem);
+  dsd_store<Cfg, 128, SCATTER>(acc, g, bi, n0, smem);
   if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <class Fused, class Triple, class Single, bool TRANS_A>
+template <class Fused, class Triple, class Single, bool TRANS_A, bool SCATTER = false>
 __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists plan, TailArgs t) {
   extern __shared__ __align__(16) char smem[];
   __shared__ int flag;
@@ -256,13 +257,13 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   const int ordinal = item - whole;  // among the tiles of the last round: 0 .. workgroups - 1
   if (item < pair_tiles) {
     const int i = xcd_share(item, pair_tiles, spread);
-    dsd_slice<Fused, TRANS_A, 2>(g, t, const_ints(plan.list(kTallPairs))[i / ntn], (i % ntn) * Fused::TN, slice, slices, ordinal, smem, &flag);
+    dsd_slice<Fused, TRANS_A, 2, SCATTER>(g, t, const_ints(plan.list(kTallPairs))[i / ntn], (i % ntn) * Fused::TN, slice, slices, ordinal, smem, &flag);
     return;
   }
   item -= pair_tiles;
   if (item < triple_tiles) {
     const int i = xcd_share(item, triple_tiles, spread);
-    dsd_slice<Triple, TRANS_A, 3>(g, t, const_ints(plan.list(kTallTriples))[i / (2 * ntn)], (i % (2 * ntn)) * Triple::TN, slice, slices, ordinal, smem, &flag);
+    dsd_slice<Triple, TRANS_A, 3, SCATTER>(g, t, const_ints(plan.list(kTallTriples))[i / (2 * ntn)], (i % (2 * ntn)) * Triple::TN, slice, slices, ordinal, smem, &flag);
     return;
   }
   item -= triple_tiles;
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(512, 2) void dsd_sliced_kernel(DsdArgs g, PlanLists
   } else {
     i = xcd_grouped(item, single_tiles);
   }
-  dsd_slice<Single, TRANS_A, 1>(g, t, const_ints(plan.list(kTallSingles))[i / ntn], (i % ntn) * Single::TN, slice, slices, ordinal, smem, &flag);
+  dsd_slice<Single, TRANS_A, 1, SCATTER>(g, t, const_ints(plan.list(kTallSingles))[i / ntn], (i % ntn) * Single::TN, slice, slices, ordinal, smem, &flag);
 }
 
 template <class Cfg, int BLK, bool TRANS_A, bool FULL>
@@ -361,6 +362,48 @@ static void launch_dsd(const DsdArgs& g, const PlanLists& plan, const TailArgs* 
   }
 }
 
+// stk_dsd_scatter: the launches of a dsd on 128-blocks with eight wavefronts (sparse operand not transposed), with
+// the rows of the result scattered.
+template <bool BF16, bool BK, bool STREAM>
+static void launch_dsd_scatter(const DsdArgs& g, const PlanLists& plan, const TailArgs* tail, hipStream_t stream) {
+  constexpr int KT = BK ? STK_DSD_BK_KT : STK_DSD_KT, S = BK ? STK_DSD_BK_STAGES : STK_DSD_STAGES;
+  using Fused = TileCfg<4, 2, 2, 4, 1, 2, 2, true, BK, BF16, KT, S, false, STREAM>;
+  using Single = TileCfg<2, 4, 2, 2, 1, 1, 2, true, BK, BF16, KT, S, false, STREAM>;
+  using Triple = TileCfg<4, 2, 3, 2, 1, 3, 1, true, BK, BF16, KT, S, false, STREAM>;
+  constexpr int lds0 = Fused::kSmemBytes > Single::kSmemBytes ? Fused::kSmemBytes : Single::kSmemBytes;
+  constexpr int lds = lds0 > Triple::kSmemBytes ? lds0 : Triple::kSmemBytes;
+  if (tail) {
+    static const int once = (set_lds_limit(&dsd_sliced_kernel<Fused, Triple, Single, false, true>, lds), 0);
+    (void)once;
+    const int grid = g.block_rows * (g.n / Fused::TN) + kMaxTailSlices * (tail->workgroups + kTailBlock);
+    hipLaunchKernelGGL((dsd_sliced_kernel<Fused, Triple, Single, false, true>), dim3(grid), dim3(512), lds, stream, g, plan, *tail);
+    return;
+  }
+  static const int once = (set_lds_limit(&dsd_fused_kernel<Fused, Triple, Single, false, true>, lds), 0);
+  (void)once;
+  hipLaunchKernelGGL((dsd_fused_kernel<Fused, Triple, Single, false, true>), dim3(g.block_rows * (g.n / Fused::TN)), dim3(512), lds, stream, g, plan);
+}
+
+// The sliced last round of a dsd launch, if this one gets one: for launches of a few rounds of tiles (with many
+// rounds the last one matters little and the plain kernel is used as it is); the plan says whether and how the last
+// round is cut.  STK_OK with *sliced set or cleared.
+static int tail_of(const char* who, const DsdArgs& g, int64_t n, int64_t nnz, int blocking, const uint8_t* plan, void* workspace,
+                   int64_t workspace_bytes, TailArgs* tail, bool* sliced) {
+  *sliced = false;
+  if (!(workspace && plan && blocking == 128 && n % 256 == 0 && nnz > 0 && !g.small)) return STK_OK;
+  const int workgroups = compute_units();
+  if (workgroups <= 0 || (int64_t)g.block_rows * (n / 128) / 3 >= 8 * (int64_t)workgroups) return STK_OK;
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(STK_ERR_WORKSPACE, "%s: the workspace must be 256-byte aligned", who);
+  const int64_t capacity = (workspace_bytes - (int64_t)tail_counter_bytes(workgroups)) / (int64_t)(sizeof(float) * kSlotFloats);
+  if (capacity < 2) return STK_OK;
+  *sliced = true;
+  tail->counters = static_cast<int32_t*>(workspace);
+  tail->slots = reinterpret_cast<float*>(static_cast<char*>(workspace) + tail_counter_bytes(workgroups));
+  tail->workgroups = workgroups;
+  tail->capacity = (int)(capacity < kMaxTailSlices * (int64_t)workgroups ? capacity : kMaxTailSlices * (int64_t)workgroups);
+  return STK_OK;
+}
+
 }  // namespace stk
 
 // Checks the arguments of a dsd and turns them into the kernels' view of the problem.  STK_OK with p->empty set when
@@ -404,6 +447,9 @@ int stk::dsd_problem(const char* who, int64_t m, int64_t k, int64_t n,
   g.block_rows = (int)block_rows;
   g.n = (int)n;
   g.idx32 = index_dtype == STK_I32;
+  g.row_map = nullptr;
+  g.row_scale = nullptr;
+  g.out_rows = 0;
   // a dense-operand row panel (one block of k) is read once per tile that walks a block in that block column of
   // op(S): with few blocks per column (a block-diagonal MoE layout has one fused tile per expert) it is streamed
   // (row-major rhs only: a K-major tile uses half a cache line per K-tile and needs the line to stay)
@@ -446,25 +492,10 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
   const DsdArgs& g = problem.g;
   const PlanLists& lists = problem.lists;
   const bool ta = problem.ta, bk = problem.bk, stream_rhs = problem.stream_rhs;
-  const int64_t block_rows = g.block_rows;
-  // Sliced last round: for launches of a few rounds of tiles (with many rounds the last one matters little and
-  // the plain kernel is used as it is); the plan says whether and how the last round is cut.
   TailArgs tail{};
   bool sliced = false;
-  if (workspace && plan && blocking == 128 && n % 256 == 0 && nnz > 0 && !g.small) {
-    const int workgroups = compute_units();
-    if (workgroups > 0 && block_rows * (n / 128) / 3 < 8 * (int64_t)workgroups) {
-      if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(STK_ERR_WORKSPACE, "stk_dsd: the workspace must be 256-byte aligned");
-      const int64_t capacity = (workspace_bytes - (int64_t)tail_counter_bytes(workgroups)) / (int64_t)(sizeof(float) * kSlotFloats);
-      if (capacity >= 2) {
-        sliced = true;
-        tail.counters = static_cast<int32_t*>(workspace);
-        tail.slots = reinterpret_cast<float*>(static_cast<char*>(workspace) + tail_counter_bytes(workgroups));
-        tail.workgroups = workgroups;
-        tail.capacity = (int)(capacity < kMaxTailSlices * (int64_t)workgroups ? capacity : kMaxTailSlices * (int64_t)workgroups);
-      }
-    }
-  }
+  const int tail_rc = tail_of("stk_dsd", g, n, nnz, blocking, plan, workspace, workspace_bytes, &tail, &sliced);
+  if (tail_rc != STK_OK) return tail_rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define STK_DSD_CASE(BF, BLK, TA, BK)                                                          \
   if ((dtype == STK_BF16) == BF && blocking == BLK && ta == TA && bk == BK) {                  \
@@ -476,6 +507,47 @@ extern "C" int stk_dsd(int64_t m, int64_t k, int64_t n,
   STK_DSD_CASE(BF, BLK, true, true) STK_DSD_CASE(BF, BLK, true, false) STK_DSD_CASE(BF, BLK, false, true) STK_DSD_CASE(BF, BLK, false, false)
   STK_DSD_LAYOUTS(true, 128) STK_DSD_LAYOUTS(false, 128) STK_DSD_LAYOUTS(true, 64) STK_DSD_LAYOUTS(false, 64)
   return fail(STK_ERR_UNSUPPORTED, "stk_dsd: no kernel for this configuration");
+}
+
+extern "C" int stk_dsd_scatter(int64_t m, int64_t k, int64_t n, const void* data, const int32_t* offsets, const void* column_indices,
+                               const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                               const int32_t* row_slots, const float* weights, int64_t num_tokens, void* out, int64_t out_stride_m,
+                               int64_t nnz, int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                               void* workspace, int64_t workspace_bytes, stk_stream_t stream) {
+  using namespace stk;
+  const char* who = "stk_dsd_scatter";
+  if (blocking != 128) return fail(STK_ERR_UNSUPPORTED, "%s: blocking %d (128 only)", who, blocking);
+  if (num_tokens < 0 || num_tokens > INT32_MAX) return fail(STK_ERR_DIMS, "%s: %lld tokens", who, (long long)num_tokens);
+  DsdProblem problem;
+  const int rc = dsd_problem(who, m, k, n, data, offsets, column_indices, nullptr, nullptr, nullptr, 0, rhs, rhs_stride_k, rhs_stride_n, out,
+                             out_stride_m, nnz, blocking, dtype, index_dtype, plan, &problem);
+  if (rc != STK_OK || problem.empty || num_tokens == 0) return rc;
+  if (!row_slots) return fail(STK_ERR_DIMS, "%s: missing row_slots", who);
+  if (n % 256 || problem.g.small)
+    return fail(STK_ERR_UNSUPPORTED, "%s: needs a multiple of 256 columns and at least %lld blocks x 128 columns per compute unit", who,
+                (long long)kSmallWorkPerUnit);
+  DsdArgs g = problem.g;
+  g.row_map = row_slots;
+  g.row_scale = weights;
+  g.out_rows = (int)num_tokens;
+  TailArgs tail{};
+  bool sliced = false;
+  const int tail_rc = tail_of(who, g, n, nnz, blocking, plan, workspace, workspace_bytes, &tail, &sliced);
+  if (tail_rc != STK_OK) return tail_rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const TailArgs* t = sliced ? &tail : nullptr;
+  const bool bf = dtype == STK_BF16;
+  if (problem.bk) {
+    if (bf) launch_dsd_scatter<true, true, false>(g, problem.lists, t, s);
+    else launch_dsd_scatter<false, true, false>(g, problem.lists, t, s);
+  } else if (problem.stream_rhs) {
+    if (bf) launch_dsd_scatter<true, false, true>(g, problem.lists, t, s);
+    else launch_dsd_scatter<false, false, true>(g, problem.lists, t, s);
+  } else {
+    if (bf) launch_dsd_scatter<true, false, false>(g, problem.lists, t, s);
+    else launch_dsd_scatter<false, false, false>(g, problem.lists, t, s);
+  }
+  return check_launch(who);
 }
 
 extern "C" int64_t stk_dsd_workspace_counter_bytes(void) {

@@ -19,6 +19,11 @@ struct DsdArgs {
   int n;
   int idx32;
   int small;       // little work per compute unit: four-wave tiles
+  // scattered output rows (the SCATTER kernels): row r of the product goes to row row_map[r] of `out`, multiplied by
+  // row_scale[row_map[r]] when row_scale is given; rows whose entry is not in [0, out_rows) are dropped
+  const int32_t* row_map;
+  const float* row_scale;
+  int out_rows;
 };
 
 // A checked dsd: the kernels' arguments, the plan's lists of the walked lines (null without a plan), layout flags.
@@ -78,21 +83,25 @@ __device__ __forceinline__ void dsd_accumulate(f32x16_t (&acc)[Cfg::IM][Cfg::JN]
 }
 
 // Writes the finished tile: the first `rows` rows from block row `bi` onwards, columns from n0.
-template <class Cfg, int BLK>
+template <class Cfg, int BLK, bool SCATTER = false>
 __device__ __forceinline__ void dsd_store(f32x16_t (&acc)[Cfg::IM][Cfg::JN], const DsdArgs& g, int bi, int n0, char* smem, int rows = Cfg::TM) {
   const int n_valid = (g.n - n0 < Cfg::TN) ? g.n - n0 : Cfg::TN;
   const WaveCoords w = wave_coords<Cfg>();
   const int wm0 = wave_m0<Cfg>(w), wn0 = wave_n0<Cfg>(w);
-  epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, rows - wm0, n_valid - wn0, smem);
+  if constexpr (SCATTER)
+    epilogue<Cfg, STK_STREAM_STORES, true>(acc, g.out + n0 + wn0, g.ldc, rows - wm0, n_valid - wn0, smem, 64, kNoActivation, nullptr, 0, 0,
+                                           g.row_map + (int64_t)bi * BLK + wm0, g.row_scale, g.out_rows);
+  else
+    epilogue<Cfg, STK_STREAM_STORES>(acc, g.out + ((int64_t)bi * BLK + wm0) * g.ldc + n0 + wn0, g.ldc, rows - wm0, n_valid - wn0, smem);
 }
 
 // The whole tile of LINES block rows starting at `bi` (the first `lines` of them exist), output columns
 // [n0, n0 + Cfg::TN).
-template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES>
+template <class Cfg, int BLK, bool TRANS_A, bool FULL, int LINES, bool SCATTER = false>
 __device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char* smem, int lines = LINES) {
   f32x16_t acc[Cfg::IM][Cfg::JN] = {};
   dsd_accumulate<Cfg, BLK, TRANS_A, FULL, LINES>(acc, g, bi, n0, 0, g.walk_offsets[bi + 1] - g.walk_offsets[bi], smem, lines);
-  dsd_store<Cfg, BLK>(acc, g, bi, n0, smem, lines * BLK);
+  dsd_store<Cfg, BLK, SCATTER>(acc, g, bi, n0, smem, lines * BLK);
 }
 
 // The tile of a launch over the plan's lists of lines (128-blocks, eight wavefronts) that workgroup `bid` takes,
@@ -102,7 +111,7 @@ __device__ __forceinline__ void dsd_tile(const DsdArgs& g, int bi, int n0, char*
 //                             are long, is still read only once for the three
 //   lone rows                 128x256 tiles
 // False when the lists have fewer tiles than that; bid then counts on past them.
-template <class Fused, class Triple, class Single, bool TRANS_A>
+template <class Fused, class Triple, class Single, bool TRANS_A, bool SCATTER = false>
 __device__ __forceinline__ bool dsd_plan_tile(const DsdArgs& g, const PlanLists& plan, int& bid, char* smem) {
   static_assert(Fused::TN == Single::TN && Fused::TN == 2 * Triple::TN, "same column tiling");
   const int ntn = g.n / Fused::TN;
@@ -111,20 +120,20 @@ __device__ __forceinline__ bool dsd_plan_tile(const DsdArgs& g, const PlanLists&
   const int single_tiles = const_ints(plan.counts)[kTallSingles] * ntn;
   if (bid < pair_tiles) {
     const int item = xcd_item(bid, pair_tiles, ntn, plan.group(kTallPairs));
-    dsd_tile<Fused, 128, TRANS_A, true, 2>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
+    dsd_tile<Fused, 128, TRANS_A, true, 2, SCATTER>(g, const_ints(plan.list(kTallPairs))[item / ntn], (item % ntn) * Fused::TN, smem);
     return true;
   }
   bid -= pair_tiles;
   if (bid < triple_tiles) {
     const int item = xcd_item(bid, triple_tiles, 2 * ntn, plan.group(kTallTriples));
-    dsd_tile<Triple, 128, TRANS_A, true, 3>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
+    dsd_tile<Triple, 128, TRANS_A, true, 3, SCATTER>(g, const_ints(plan.list(kTallTriples))[item / (2 * ntn)], (item % (2 * ntn)) * Triple::TN, smem);
     return true;
   }
   bid -= triple_tiles;
   if (bid < single_tiles) {
     // (in order of length: no contiguous shares; by stripes of the dense operand when the plan says so, in its 256-wide tiles)
     const int item = xcd_lines(bid, single_tiles, ntn, (plan.stripe_from(true) + 1) >> 1);
-    dsd_tile<Single, 128, TRANS_A, true, 1>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
+    dsd_tile<Single, 128, TRANS_A, true, 1, SCATTER>(g, const_ints(plan.list(kTallSingles))[item / ntn], (item % ntn) * Single::TN, smem);
     return true;
   }
   bid -= single_tiles;

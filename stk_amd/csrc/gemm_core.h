@@ -39,6 +39,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace stk {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -85,6 +87,16 @@ template <bool BF16>
 __device__ __forceinline__ uint32_t mul_packed(uint32_t a, uint32_t b) {
   const f32x2_t x = unpack2<BF16>(a), y = unpack2<BF16>(b);
   return pack2<BF16>(x.x * y.x, x.y * y.y);
+}
+// A packed pair times an fp32 factor: the product rounded to fp32, then to 16 bits.
+template <bool BF16>
+__device__ __forceinline__ uint32_t scale_packed(uint32_t a, float w) {
+  const f32x2_t x = unpack2<BF16>(a);
+  float lo = w * x.x, hi = w * x.y;
+  // (final fp32 values: otherwise the multiplication and the conversion may become one mixed-precision
+  // instruction that does not round the product to fp32 first)
+  asm volatile("" : "+v"(lo), "+v"(hi));
+  return pack2<BF16>(lo, hi);
 }
 
 // Activation functions that a product can apply to its fp32 accumulators before they are rounded.
@@ -230,6 +242,18 @@ struct Operand {
   __device__ __forceinline__ static void dma_offsets(uint32_t (&off)[kSlicesPerWave], int wave, int lane, int64_t ld) {
 #pragma unroll
     for (int i = 0; i < kSlicesPerWave; i++) off[i] = dma_lane_offset(i * kWaves + wave, lane, ld);
+  }
+  // The same for a K-major operand whose rows are gathered: row `row` of the tile is row source_row(row) of the
+  // array at the tile origin (which then is the array's first row at the K-tile's k).
+  template <class SourceRow>
+  __device__ __forceinline__ static void dma_offsets_gathered(uint32_t (&off)[kSlicesPerWave], int wave, int lane, int64_t ld, SourceRow&& source_row) {
+    static_assert(KMAJOR, "rows are gathered, not columns");
+#pragma unroll
+    for (int i = 0; i < kSlicesPerWave; i++) {
+      const int row = (i * kWaves + wave) * (1024 / (KT * 2)) + lane / kCR;
+      const int chunk = (lane % kCR) ^ kmajor_swizzle(row);
+      off[i] = (uint32_t)(((int64_t)source_row(row) * ld + chunk * 8) * 2);
+    }
   }
 
   // ---- register path --------------------------------------------------------
@@ -435,9 +459,13 @@ __device__ __forceinline__ void static_for(Fn&& fn) {
 // K-tile t; it is called exactly once per t, in increasing order.
 // after_prologue() runs once, behind the transfers of the first STAGES - 1 K-tiles and in front of the first wait: work
 // that does not depend on the tile (the caller's look-ahead) sits there in the shadow of the first transfers' latency.
-template <class Cfg, class TileFn, class Hook>
+// rows_a(q, row): the row of the array at part q's origin that holds row `row` of that part of the A tile
+// (ConsecutiveRows: the rows follow each other from the origin; anything else needs a K-major A operand and offsets
+// of less than 4 GiB from the origin).
+struct ConsecutiveRows {};
+template <class Cfg, class TileFn, class Hook, class RowsA>
 __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
-                                             int64_t lda, int64_t ldb, char* smem, Hook&& after_prologue) {
+                                             int64_t lda, int64_t ldb, char* smem, Hook&& after_prologue, RowsA&& rows_a) {
   using OpA = typename Cfg::OpA;
   using OpB = typename Cfg::OpB;
   constexpr int S = Cfg::STAGES;
@@ -447,8 +475,14 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
   const WaveCoords w = wave_coords<Cfg>();
   const uint32_t lds0 = (uint32_t)(uintptr_t)((STK_LDS char*)smem);
 
-  uint32_t offa[OpA::kSlicesPerWave], offb[OpB::kSlicesPerWave];
-  OpA::dma_offsets(offa, w.wave, w.lane, lda);
+  constexpr bool kGathered = !std::is_same<typename std::decay<RowsA>::type, ConsecutiveRows>::value;
+  uint32_t offa[kGathered ? Cfg::A_PARTS : 1][OpA::kSlicesPerWave], offb[OpB::kSlicesPerWave];
+  if constexpr (kGathered) {
+#pragma unroll
+    for (int q = 0; q < Cfg::A_PARTS; q++) OpA::dma_offsets_gathered(offa[q], w.wave, w.lane, lda, [&](int row) { return rows_a(q, row); });
+  } else {
+    OpA::dma_offsets(offa[0], w.wave, w.lane, lda);
+  }
   OpB::dma_offsets(offb, w.wave, w.lane, ldb);
   // The loads of K-tile t in two steps: the operand origins as scalar pointers (address arithmetic that can
   // run in the shadow of MFMAs), then the transfers themselves, one 1 KiB piece per call.
@@ -469,7 +503,7 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
     constexpr int P = decltype(piece)::value;
     if constexpr (P < kLoadsA) {
       constexpr int q = P / OpA::kSlicesPerWave, i = P % OpA::kSlicesPerWave;
-      dma16<Cfg::STREAM_A>(o.a[q], offa[i], stage + q * OpA::kBytes + (i * OpA::kWaves + w.wave) * 1024);
+      dma16<Cfg::STREAM_A>(o.a[q], offa[kGathered ? q : 0][i], stage + q * OpA::kBytes + (i * OpA::kWaves + w.wave) * 1024);
     } else if constexpr (P < kLoadsPerTile) {
       constexpr int q = (P - kLoadsA) / OpB::kSlicesPerWave, i = (P - kLoadsA) % OpB::kSlicesPerWave;
       dma16<Cfg::STREAM_B>(o.b[q], offb[i], stage + Cfg::A_PARTS * OpA::kBytes + q * OpB::kBytes + (i * OpB::kWaves + w.wave) * 1024);
@@ -594,10 +628,15 @@ __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
   }
   __syncthreads();  // operand reads done before the epilogue reuses LDS
 }
+template <class Cfg, class TileFn, class Hook>
+__device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
+                                             int64_t lda, int64_t ldb, char* smem, Hook&& after_prologue) {
+  mainloop_dma<Cfg>(acc, ntiles, tile_fn, lda, ldb, smem, after_prologue, ConsecutiveRows{});
+}
 template <class Cfg, class TileFn>
 __device__ __forceinline__ void mainloop_dma(f32x16_t (&acc)[Cfg::IM][Cfg::JN], int ntiles, TileFn&& tile_fn,
                                              int64_t lda, int64_t ldb, char* smem) {
-  mainloop_dma<Cfg>(acc, ntiles, tile_fn, lda, ldb, smem, [] {});
+  mainloop_dma<Cfg>(acc, ntiles, tile_fn, lda, ldb, smem, [] {}, ConsecutiveRows{});
 }
 
 // Ragged tiles: predicated register staging, two LDS stages.
@@ -654,11 +693,16 @@ __device__ __forceinline__ void mainloop_reg(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
 // activation (wave-uniform): applied to the fp32 sums before they are rounded.
 // mul (wave-uniform, or null): an array laid out like `out`, pointing at the same element; the rounded
 // values are multiplied by its elements and rounded again.
-template <class Cfg, bool STREAM>
+// SCATTER: row gm of the sub-tile goes to row row_map[gm] of the array whose row 0 `out` then points into (at the
+// sub-tile's first column); rows whose entry is negative or not below out_rows are dropped.  row_scale (or null):
+// fp32 factors by destination row; the rounded values are multiplied by them and rounded again.
+template <class Cfg, bool STREAM, bool SCATTER = false>
 __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem_t* out, int64_t ldc,
                                          int m_valid, int n_valid, char* smem, int64_t quadrant_stride = 64,
                                          int activation = kNoActivation, const elem_t* mul = nullptr,
-                                         int row_base = 0, int64_t row_jump = 0) {
+                                         int row_base = 0, int64_t row_jump = 0, const int32_t* row_map = nullptr,
+                                         const float* row_scale = nullptr, int out_rows = 0) {
+  static_assert(!SCATTER || Cfg::WK == 1, "scattered rows: whole-K wavefront tiles only");
   // (the thread's id through an opaque statement: in a workgroup that loops over tiles the store addresses below would
   // otherwise be computed once in front of the loop and held in registers through every K loop)
   int tid = threadIdx.x;
@@ -679,6 +723,20 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
           gm = qi * 64 + m, gn = qj * 64 + ch * 8;
           return (int64_t)gm * ldc + qj * quadrant_stride + ch * 8 + (int64_t)((row_base + gm) >> 7) * row_jump;
         };
+        // scattered rows: where this pass's rows go and what they are scaled by, read once
+        int dest[SCATTER ? 8 : 1];
+        float scale[SCATTER ? 8 : 1];
+        if constexpr (SCATTER) {
+#pragma unroll
+          for (int it = 0; it < 8; it++) {
+            const int gm = qi * 64 + it * 8 + (lane >> 3);
+            int d = -1;
+            if (it < 4 * strips && gm < m_valid) d = row_map[gm];
+            dest[it] = d < out_rows ? d : -1;
+          }
+#pragma unroll
+          for (int it = 0; it < 8; it++) scale[it] = (row_scale && dest[it] >= 0) ? row_scale[dest[it]] : 1.0f;
+        }
         // the multiplier's values of this pass, read once: on their way while the sums are rounded and staged
         u32x4 factor[8];
         if (mul) {
@@ -720,11 +778,22 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
           u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4));
           if ((m >> 4) & 1) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
           int gm, gn;
-          const int64_t at = place(it, gm, gn);
-          if (gm < m_valid && gn < n_valid) {
+          int64_t at = place(it, gm, gn);
+          bool wanted = gm < m_valid && gn < n_valid;
+          if constexpr (SCATTER) {
+            wanted = wanted && dest[it] >= 0;
+            at = (int64_t)dest[it] * ldc + gn;
+          }
+          if (wanted) {
             if (mul) {
               const u32x4 f = factor[it];
               v = u32x4{mul_packed<Cfg::BF16>(v.x, f.x), mul_packed<Cfg::BF16>(v.y, f.y), mul_packed<Cfg::BF16>(v.z, f.z), mul_packed<Cfg::BF16>(v.w, f.w)};
+            }
+            if constexpr (SCATTER) {
+              if (row_scale) {
+                const float f = scale[it];
+                v = u32x4{scale_packed<Cfg::BF16>(v.x, f), scale_packed<Cfg::BF16>(v.y, f), scale_packed<Cfg::BF16>(v.z, f), scale_packed<Cfg::BF16>(v.w, f)};
+              }
             }
             u32x4* dst = reinterpret_cast<u32x4*>(out + at);
             if constexpr (STREAM) __builtin_nontemporal_store(v, dst);

@@ -20,34 +20,7 @@ namespace stk {
 template <class Quad, class Pair, class Triple, bool FULL>
 __global__ __launch_bounds__(512, 2) void sdd_fused_kernel(SddArgs g) {
   extern __shared__ __align__(16) char smem[];
-  if (g.tiles) {
-    const int count = const_ints(g.tiles)[0];
-    if ((int)blockIdx.x >= count) return;
-    const int item = xcd_tile(blockIdx.x, count);
-    sdd_plan_tile<Quad, Pair, Triple, FULL>(g, item, smem);
-    return;
-  }
-  const int npairs = (g.nnz + 1) >> 1;
-  const int q = xcd_chunked(blockIdx.x, npairs);
-  const int p0 = 2 * q;
-  const bool has1 = p0 + 1 < g.nnz;
-  const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
-  const int r1 = has1 ? uniform(load_index(g.row_indices, p0 + 1, g.idx32)) : -1;
-  const int c0 = uniform(load_index(g.column_indices, p0, g.idx32));
-  const int c1 = has1 ? uniform(load_index(g.column_indices, p0 + 1, g.idx32)) : c0;
-  if (r1 != r0) {
-    // the two blocks lie in different rows (or the second does not exist): one at a time
-#pragma unroll 1
-    for (int i = 0; i < (has1 ? 2 : 1); i++) {
-      const int r = i ? r1 : r0, c = i ? c1 : c0;
-      const int rr[3] = {r, r, r}, cc[2] = {c, c}, pp[3][2] = {{p0 + i, -1}, {-1, -1}, {-1, -1}};
-      sdd_tile<Pair, 128, FULL>(g, rr, cc, pp, smem);
-      __syncthreads();  // the epilogue staging buffer is part of the next pass's first stage
-    }
-    return;
-  }
-  const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, p0 + 1}, {-1, -1}, {-1, -1}};
-  sdd_tile<Pair, 128, FULL>(g, rr, cc, pp, smem);
+  sdd_fused_tile<Quad, Pair, Triple, FULL>(g, smem);
 }
 
 // 64-blocks with a plan: a tile of up to 4 x 4 blocks.  rows identical block rows starting at r0 (their

@@ -23,19 +23,33 @@ struct SddArgs {
   int idx32;
   int activation;            // applied to the fp32 sums (an Activation value)
   const elem_t* multiplier;  // values of a matrix with the same topology, multiplied in after the rounding; or null
+  // gathered lhs rows (the GATHER kernels): row r of the lhs is row row_slots[r] / top_k of `lhs`, a row of zeros
+  // where row_slots[r] is not in [0, slots)
+  const int32_t* row_slots;
+  int top_k;
+  int slots;
 };
+
+// The row of SddArgs::lhs that row `r` of a gathered lhs is taken from; negative: a row of zeros.
+__device__ __forceinline__ int gathered_row(const SddArgs& g, int r) {
+  const int s = g.row_slots[r];
+  return (s < 0 || s >= g.slots) ? -1 : s / g.top_k;
+}
 
 // A tile of Cfg::A_PARTS block rows x Cfg::B_PARTS block columns.  r[i] / c[j] are the
 // block rows / columns, p[i][j] the output block ids (negative: not stored).
-template <class Cfg, int BLK, bool FULL>
+// GATHER: the rows of the lhs are gathered (SddArgs::row_slots); the transfers of the lhs tiles then take every row
+// from where it lies, and rows of zeros are computed on the array's first row and set to zero afterwards.
+template <class Cfg, int BLK, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem) {
   static_assert(Cfg::PM == BLK && Cfg::PN == BLK && Cfg::A_PARTS <= 3 && Cfg::B_PARTS <= 2, "one operand part per block row / column");
+  static_assert(!GATHER || (FULL && Cfg::A_KMAJOR), "gathered rows: row-major lhs, direct-to-LDS pipeline");
   constexpr int KT = Cfg::KT;
   // K-major: ld is the stride between rows of the tile; MN-major: between k rows.
   const elem_t* a0[3];
   const elem_t* b0[2];
 #pragma unroll
-  for (int i = 0; i < 3; i++) a0[i] = g.lhs + (int64_t)r[i] * BLK * (Cfg::A_KMAJOR ? g.lda : 1);
+  for (int i = 0; i < 3; i++) a0[i] = GATHER ? g.lhs : g.lhs + (int64_t)r[i] * BLK * (Cfg::A_KMAJOR ? g.lda : 1);
 #pragma unroll
   for (int j = 0; j < 2; j++) b0[j] = g.rhs + (int64_t)c[j] * BLK * (Cfg::B_KMAJOR ? g.ldb : 1);
   const int64_t a_step = Cfg::A_KMAJOR ? KT : KT * g.lda;
@@ -47,10 +61,31 @@ __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], co
     const int left = k - t * KT;
     return TilePtrs{{a0[0] + t * a_step, a0[1] + t * a_step, a0[2] + t * a_step}, {b0[0] + t * b_step, b0[1] + t * b_step}, left < KT ? left : KT};
   };
-  if constexpr (FULL) mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem);
-  else mainloop_reg<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, BLK, BLK, smem);
+  if constexpr (GATHER) {
+    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem, [] {}, [&](int q, int row) {
+      const int from = gathered_row(g, r[q] * BLK + row);
+      return from < 0 ? 0 : from;
+    });
+  } else if constexpr (FULL) {
+    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem);
+  } else {
+    mainloop_reg<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, BLK, BLK, smem);
+  }
   const WaveCoords w = wave_coords<Cfg>();
   const int m0 = wave_m0<Cfg>(w), n0 = wave_n0<Cfg>(w);
+  if constexpr (GATHER) {
+    // lane l holds row 32 i + l % 32 of the wavefront's sub-tile in acc[i][..]
+#pragma unroll
+    for (int i = 0; i < Cfg::IM; i++) {
+      const int m = m0 + 32 * i + (w.lane & 31);
+      const int part = m / BLK;
+      const int br = part == 0 ? r[0] : (part == 1 ? r[1] : r[2]);
+      if (gathered_row(g, br * BLK + m % BLK) < 0) {
+#pragma unroll
+        for (int j = 0; j < Cfg::JN; j++) acc[i][j] = f32x16_t{};
+      }
+    }
+  }
   if constexpr (Cfg::A_PARTS == 3) {
     // Three stored blocks below each other, one block wide; a wavefront's 96 rows may lie in two of them.
     // Addressed as rows of the first block that run on, with the distance between the blocks added per block.
@@ -68,7 +103,7 @@ __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], co
 // The tile `item` of the plan's list (128-blocks): two neighbouring blocks of a block row (1x2 blocks, 128x256),
 // together with the two blocks below when the next row repeats this one (2x2 blocks, 256x256), or one block with
 // the two below it for the last three rows of a run of odd length (3x1 blocks, 384x128).
-template <class Quad, class Pair, class Triple, bool FULL>
+template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* smem) {
   const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
   const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
@@ -80,14 +115,48 @@ __device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* 
   if (rows == 3) {
     // the last three rows of a run of identical rows: one block wide, so that the rhs panel is read once for the three
     const int rr[3] = {r0, r0 + 1, r0 + 2}, cc[2] = {c0, c0}, pp[3][2] = {{p0, -1}, {below, -1}, {below + nseg, -1}};
-    sdd_tile<Triple, 128, FULL>(g, rr, cc, pp, smem);
+    sdd_tile<Triple, 128, FULL, GATHER>(g, rr, cc, pp, smem);
   } else if (below >= 0) {
     const int rr[3] = {r0, r0 + 1, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {below, has1 ? below + 1 : -1}, {-1, -1}};
-    sdd_tile<Quad, 128, FULL>(g, rr, cc, pp, smem);
+    sdd_tile<Quad, 128, FULL, GATHER>(g, rr, cc, pp, smem);
   } else {
     const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {-1, -1}, {-1, -1}};
-    sdd_tile<Pair, 128, FULL>(g, rr, cc, pp, smem);
+    sdd_tile<Pair, 128, FULL, GATHER>(g, rr, cc, pp, smem);
   }
+}
+
+// What workgroup blockIdx.x of a launch over 128-blocks with eight wavefronts computes: its tile of the plan's list,
+// or without a plan the blockIdx.x-th pair of blocks in CSR order (every row on its own).
+template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
+__device__ __forceinline__ void sdd_fused_tile(const SddArgs& g, char* smem) {
+  if (g.tiles) {
+    const int count = const_ints(g.tiles)[0];
+    if ((int)blockIdx.x >= count) return;
+    const int item = xcd_tile(blockIdx.x, count);
+    sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, item, smem);
+    return;
+  }
+  const int npairs = (g.nnz + 1) >> 1;
+  const int q = xcd_chunked(blockIdx.x, npairs);
+  const int p0 = 2 * q;
+  const bool has1 = p0 + 1 < g.nnz;
+  const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
+  const int r1 = has1 ? uniform(load_index(g.row_indices, p0 + 1, g.idx32)) : -1;
+  const int c0 = uniform(load_index(g.column_indices, p0, g.idx32));
+  const int c1 = has1 ? uniform(load_index(g.column_indices, p0 + 1, g.idx32)) : c0;
+  if (r1 != r0) {
+    // the two blocks lie in different rows (or the second does not exist): one at a time
+#pragma unroll 1
+    for (int i = 0; i < (has1 ? 2 : 1); i++) {
+      const int r = i ? r1 : r0, c = i ? c1 : c0;
+      const int rr[3] = {r, r, r}, cc[2] = {c, c}, pp[3][2] = {{p0 + i, -1}, {-1, -1}, {-1, -1}};
+      sdd_tile<Pair, 128, FULL, GATHER>(g, rr, cc, pp, smem);
+      __syncthreads();  // the epilogue staging buffer is part of the next pass's first stage
+    }
+    return;
+  }
+  const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, p0 + 1}, {-1, -1}, {-1, -1}};
+  sdd_tile<Pair, 128, FULL, GATHER>(g, rr, cc, pp, smem);
 }
 
 // A checked sdd: the kernels' arguments and the operands' layouts.

@@ -9,6 +9,7 @@ from collections import namedtuple
 import torch
 
 from stk_amd.backend import hip_kernels
+from stk_amd.matrix import Matrix
 
 Route = namedtuple("Route", "indices bin_ids bins padded_bins slot_rows row_slots top_k blocking")
 
@@ -83,3 +84,40 @@ def padded_scatter(x, route, weights=None):
     """x [padded_rows, hidden] -> [tokens, hidden]: each token's top_k rows, multiplied by
     weights [tokens, top_k] (or [tokens * top_k]) when given, added up in fp32 in the order of the choices."""
     return _PaddedScatter.apply(x, route, weights)
+
+
+def _wants_grad(*tensors):
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def gather_sdd(x, route, rhs, topo, activation=None):
+    """stk.ops.sdd_fused(padded_gather(x, route), rhs, topo, activation) in one launch: the sampled product reads the
+    token rows where they lie, and the padded copy of x is never made.  The result is bit-identical to the two steps.
+    Used when nothing needs a gradient (the backward pass of the product needs the padded copy anyway) and the library
+    has the kernel (128-blocks); otherwise the two steps run."""
+    from stk_amd.ops import linear_ops
+    assert isinstance(topo, Matrix) and topo.is_contiguous()
+    if x.is_cuda and not _wants_grad(x, rhs):
+        out = torch.empty_like(topo.data)
+        if hip_kernels.sdd_gather(x, route.row_slots, route.top_k, rhs, topo.size(), out, topo.offsets, topo.row_indices, topo.column_indices,
+                                  activation):
+            return Matrix(topo.size(), out, topo.row_indices, topo.column_indices, topo.offsets,
+                          topo.column_indices_t, topo.offsets_t, topo.block_offsets_t)
+    return linear_ops.sdd_fused(padded_gather(x, route), rhs, topo, activation)
+
+
+def dsd_scatter(a, rhs, route, weights=None):
+    """padded_scatter(stk.ops.dsd(a, rhs), route, weights) in one launch for top_k = 1: the product's store writes
+    every row to its token's place (times its weight), and the padded result is never made.  The result is
+    bit-identical to the two steps.  Used when nothing needs a gradient, the routing is top-1 and the library has the
+    kernel (128-blocks, a multiple of 256 columns, enough work for the eight-wavefront tiles); otherwise the two steps
+    run."""
+    from stk_amd.ops import linear_ops
+    assert isinstance(a, Matrix)
+    if route.top_k == 1 and a.is_contiguous() and a.data.is_cuda and not _wants_grad(a.data, rhs, weights):
+        tokens = route.slot_rows.numel()
+        out = torch.empty((tokens, rhs.shape[1]), dtype=a.dtype, device=a.data.device)
+        if hip_kernels.dsd_scatter(a.size(), a.data, a.offsets, a.column_indices, a.offsets_t, a.column_indices_t, rhs,
+                                   route.row_slots, weights, out):
+            return out
+    return padded_scatter(linear_ops.dsd(a, rhs), route, weights)
