@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define STK_AMD_ABI_VERSION 15
+#define STK_AMD_ABI_VERSION 16
 
 /* status codes */
 #define STK_OK 0
@@ -162,6 +162,32 @@ int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
                   const int32_t* block_order, int64_t nnz,
                   int blocking, int dtype, int index_dtype, const uint8_t* plan,
                   int activation, const void* multiplier, stk_stream_t stream);
+
+/*
+ * stk_sdd_fused that also keeps the sums: `sums` (NULL: not kept, the call is stk_sdd_fused), an array laid out like
+ * `out` and distinct from it, receives round(lhs * rhs) block by block - what stk_sdd would have stored - while `out`
+ * receives the activated and multiplied values.  A training step that keeps them gets the gradient with respect to the
+ * sums from stk_activation_product, one pass over the values, instead of from a second product that computes the sums
+ * again; it then stores what the reference's callers store (they keep the result of sdd(),
+ * stk/ops/linear_ops.py:37-59, for the backward pass of their activation).  16-bit values only.
+ */
+int stk_sdd_fused_sums(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                       const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                       int64_t m, int64_t k, int64_t n,
+                       void* out, const int32_t* offsets, const void* row_indices, const void* column_indices,
+                       const int32_t* block_order, int64_t nnz,
+                       int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                       int activation, const void* multiplier, void* sums, stk_stream_t stream);
+
+/*
+ * out[i] = round(round(act(sums[i])) * factor[i]) for i < count (factor NULL: the first rounding only): the
+ * element-wise arithmetic of stk_sdd_fused's store applied to stored 16-bit sums.  act is any STK_ACT_* code; with a
+ * derivative and the incoming gradient as `factor` this is the gradient with respect to the sums.  count a multiple
+ * of 8, arrays 16-byte aligned, `out` may be `factor` or `sums`.  Stands in for the element-wise passes that the
+ * reference's callers run in torch on the values of a Matrix (stk/ops/eltwise_ops.py:3-28 is their multiplication).
+ */
+int stk_activation_product(const void* sums, const void* factor, void* out, int64_t count, int activation, int dtype,
+                           stk_stream_t stream);
 
 /*
  * out[m, n] = op(S)[m, k] * rhs[k, n], op = transpose when transpose_a != 0.

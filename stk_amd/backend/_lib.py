@@ -11,7 +11,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstk_amd.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 STK_OK, STK_ERR_DIMS, STK_ERR_UNSUPPORTED, STK_ERR_HIP, STK_ERR_WORKSPACE = 0, 1, 2, 3, 4
 STK_F16, STK_BF16, STK_F32 = 0, 1, 2
 STK_I16, STK_I32 = 0, 1
@@ -27,6 +27,8 @@ SIGNATURES = {
     "stk_build_plan": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _int, _int, _p, _sz, _p]),
     "stk_sdd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _p]),
     "stk_sdd_fused": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _int, _p, _p]),
+    "stk_sdd_fused_sums": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i64, _int, _int, _int, _p, _int, _p, _p, _p]),
+    "stk_activation_product": (_int, [_p, _p, _p, _i64, _int, _int, _p]),
     "stk_dsd_workspace_bytes": (_i64, [_i64, _i64, _int]),
     "stk_dsd_workspace_counter_bytes": (_i64, []),
     "stk_dsd_workspace_slot_bytes": (_i64, []),

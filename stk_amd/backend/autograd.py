@@ -247,32 +247,39 @@ _FUSED_ACTIVATIONS = (None, "none", "relu", "silu", "gelu", "gelu_tanh")   # (th
 
 class SDDFused(torch.autograd.Function):
     """activation(sdd(lhs, rhs)) * multiplier in one pass (no counterpart in the reference, whose callers run
-    the activation and stk.ops.mul, stk/ops/eltwise_ops.py:3-28, as passes of their own).  Only the result is
-    stored; backward recomputes the sums in an sdd whose store applies the activation's derivative and multiplies
-    by the incoming gradient, and then follows SDD.backward."""
+    the activation and stk.ops.mul, stk/ops/eltwise_ops.py:3-28, as passes of their own).  Without save_sums only the
+    result is stored; backward recomputes the sums in an sdd whose store applies the activation's derivative and
+    multiplies by the incoming gradient.  With save_sums the forward product also stores the rounded sums (what the
+    reference's callers keep: the result of sdd() in front of their activation), and backward gets the same gradient
+    from one element-wise pass over them - less time, one more array of values.  Either way it then follows
+    SDD.backward."""
 
     @staticmethod
     @custom_fwd
     def forward(ctx, lhs, rhs, shape, data, offsets, row_indices, column_indices, offsets_t, column_indices_t,
-                block_offsets_t, activation, multiplier):
+                block_offsets_t, activation, multiplier, save_sums=False):
         if activation not in _FUSED_ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}")
         out = torch.empty(data.shape, dtype=lhs.dtype, device=lhs.device)
         values = None if multiplier is None else multiplier.detach().contiguous()
+        keep = bool(save_sums) and activation not in (None, "none") and lhs.is_cuda and any(ctx.needs_input_grad)
+        sums = torch.empty_like(out) if keep else None
         backend.prepare_plan(data, offsets, column_indices, offsets_t, column_indices_t)
         backend.sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activation, values,
-                          block_order=block_offsets_t)
+                          block_order=block_offsets_t, sums=sums)
         ctx.save_for_backward(lhs, rhs, offsets, row_indices, column_indices, offsets_t, column_indices_t,
-                              block_offsets_t, *(() if values is None else (values,)))
+                              block_offsets_t, *(() if values is None else (values,)), *(() if sums is None else (sums,)))
         ctx.shape = tuple(shape)
         ctx.activation = activation
         ctx.has_multiplier = values is not None
+        ctx.has_sums = sums is not None
         return out
 
     @staticmethod
     @custom_bwd
     def backward(ctx, dy):
         lhs, rhs, *meta = ctx.saved_tensors
+        sums = meta.pop() if ctx.has_sums else None
         values = meta.pop() if ctx.has_multiplier else None
         offsets, row_indices, column_indices, _, _, block_offsets_t = meta
         plain = ctx.activation in (None, "none")
@@ -280,6 +287,8 @@ class SDDFused(torch.autograd.Function):
             dy = dy.contiguous()
 
         def recompute(activation, multiplier):
+            if sums is not None:
+                return backend.activation_product(sums, multiplier, activation)
             out = torch.empty(dy.shape, dtype=lhs.dtype, device=lhs.device)
             backend.sdd_fused(lhs, rhs, ctx.shape, out, offsets, row_indices, column_indices, activation, multiplier,
                               block_order=block_offsets_t)
@@ -294,7 +303,7 @@ class SDDFused(torch.autograd.Function):
         g = dy if values is None else dy * values
         dsums = g if plain else recompute(ctx.activation + "_grad", g)
         dlhs, drhs = _sdd_operand_gradients(ctx, lhs, rhs, _Sparse(ctx.shape, dsums, *meta), dsums)
-        return dlhs, drhs, None, None, None, None, None, None, None, None, None, dmul
+        return dlhs, drhs, None, None, None, None, None, None, None, None, None, dmul, None
 
 
 class RowIndices(torch.autograd.Function):

@@ -226,9 +226,10 @@ def sdd(lhs, rhs, shape, out, offsets, row_indices, column_indices, block_order=
 
 
 def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activation=None, multiplier=None,
-              block_order=None):
+              block_order=None, sums=None):
     """sdd whose store applies `activation` (a key of ACTIVATIONS) to the fp32 sums and, after the
     rounding, multiplies by `multiplier` ([nnz, b, b] values of a matrix with the same topology).
+    `sums` (like `out`, or None) also receives the rounded sums themselves (stk_sdd_fused_sums).
     No counterpart as one call in the reference, whose callers run the activation and
     stk.ops.mul (stk/ops/eltwise_ops.py:3-28) as passes of their own over the values."""
     assert lhs.shape[1] == rhs.shape[0], "incompatible dimensions"
@@ -237,7 +238,7 @@ def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activa
     b = _blocking(out)
     _validate_matmul_dims(m, k, n, b)
     if not out.is_cuda:
-        if ACTIVATIONS.get(activation, 1) != 0 or multiplier is not None:
+        if ACTIVATIONS.get(activation, 1) != 0 or multiplier is not None or sums is not None:
             raise NotImplementedError("stk_amd: the fused store of sdd runs on a GPU only")
         return host_kernels.sdd(lhs, rhs, shape, out, offsets, row_indices, column_indices)
     _need_gpu(lhs, rhs, out)
@@ -248,6 +249,9 @@ def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activa
     if multiplier is not None:
         _need_gpu(multiplier)
         assert multiplier.shape == out.shape and multiplier.dtype == out.dtype and multiplier.is_contiguous()
+    if sums is not None:
+        _need_gpu(sums)
+        assert sums.shape == out.shape and sums.dtype == out.dtype and sums.is_contiguous() and sums.data_ptr() != out.data_ptr()
     if nnz == 0:
         return
     lhs, rhs = _dense_operand(lhs), _dense_operand(rhs)
@@ -260,12 +264,33 @@ def sdd_fused(lhs, rhs, shape, out, offsets, row_indices, column_indices, activa
         order = block_order.contiguous()
     plan = fusion_plan(offsets, column_indices, blocking=b) if FUSION and b in (64, 128) and offsets is not None else None
     with _on_device(out.device):
-        _lib.check(_lib.load().stk_sdd_fused(
+        _lib.check(_lib.load().stk_sdd_fused_sums(
             lhs.data_ptr(), lhs.stride(0), lhs.stride(1), rhs.data_ptr(), rhs.stride(0), rhs.stride(1),
             m, k, n, out.data_ptr(), _offsets(offsets).data_ptr() if plan is not None else None, ri.data_ptr(), ci.data_ptr(),
             order.data_ptr() if order is not None else None, nnz,
             b, _value_dtype(out), _INDEX_DTYPES[ri.dtype], plan.data_ptr() if plan is not None else None,
-            ACTIVATIONS[activation], multiplier.data_ptr() if multiplier is not None else None, _stream()))
+            ACTIVATIONS[activation], multiplier.data_ptr() if multiplier is not None else None,
+            sums.data_ptr() if sums is not None else None, _stream()))
+
+
+def activation_product(sums, factor, activation):
+    """round(round(act(sums)) * factor) over the values of a sparse matrix (factor None: the first rounding only);
+    `activation` a key of ACTIVATIONS, derivatives included (stk_activation_product)."""
+    _need_gpu(sums)
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"unknown activation {activation!r}")
+    sums = sums.detach().contiguous()
+    out = torch.empty_like(sums)
+    if factor is not None:
+        _need_gpu(factor)
+        factor = factor.detach().contiguous()
+        assert factor.shape == sums.shape and factor.dtype == sums.dtype
+    if sums.numel() == 0:
+        return out
+    with _on_device(sums.device):
+        _lib.check(_lib.load().stk_activation_product(sums.data_ptr(), factor.data_ptr() if factor is not None else None, out.data_ptr(),
+                                                      sums.numel(), ACTIVATIONS[activation], _value_dtype(sums), _stream()))
+    return out
 
 
 # dsd launches that fill the GPU only a few times cut the tiles of their last round into slices

@@ -696,12 +696,14 @@ __device__ __forceinline__ void mainloop_reg(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
 // SCATTER: row gm of the sub-tile goes to row row_map[gm] of the array whose row 0 `out` then points into (at the
 // sub-tile's first column); rows whose entry is negative or not below out_rows are dropped.  row_scale (or null):
 // fp32 factors by destination row; the rounded values are multiplied by them and rounded again.
+// sums (wave-uniform, or null): an array laid out like `out`, pointing at the same element; it receives the sums
+// rounded to 16 bits as they are, before the activation and the multiplier.
 template <class Cfg, bool STREAM, bool SCATTER = false>
 __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem_t* out, int64_t ldc,
                                          int m_valid, int n_valid, char* smem, int64_t quadrant_stride = 64,
                                          int activation = kNoActivation, const elem_t* mul = nullptr,
                                          int row_base = 0, int64_t row_jump = 0, const int32_t* row_map = nullptr,
-                                         const float* row_scale = nullptr, int out_rows = 0) {
+                                         const float* row_scale = nullptr, int out_rows = 0, elem_t* sums = nullptr) {
   static_assert(!SCATTER || Cfg::WK == 1, "scattered rows: whole-K wavefront tiles only");
   // (the thread's id through an opaque statement: in a workgroup that loops over tiles the store addresses below would
   // otherwise be computed once in front of the loop and held in registers through every K loop)
@@ -748,6 +750,44 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
             if (it < 4 * strips && gm < m_valid && gn < n_valid) factor[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mul + at));
           }
         }
+        // rounds this pass's sums to 16 bits and puts them into the staging buffer, element (m, n) of the pass's 64 x 64
+        // quadrant at row m, 8-byte unit swizzled by the row
+        auto stage = [&]() {
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+              for (int g = 0; g < 4; g++) {
+                if (i >= strips) continue;
+                const f32x16_t& c = acc[(2 * qi + i) < Cfg::IM ? 2 * qi + i : 0][2 * qj + j];
+                int m = i * 32 + (lane & 31);
+                int ch = 4 * j + g;
+                u32x2 v = {pack2<Cfg::BF16>(c[4 * g], c[4 * g + 1]), pack2<Cfg::BF16>(c[4 * g + 2], c[4 * g + 3])};
+                *reinterpret_cast<u32x2*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4) + ((((lane >> 5) ^ (m >> 4)) & 1) << 3)) = v;
+              }
+        };
+        // piece `it` of the staged pass: eight consecutive elements of a row
+        // (no barrier: the staging buffer is private to the wavefront and LDS serves a wavefront's accesses in order)
+        auto staged = [&](int it) {
+          int m = it * 8 + (lane >> 3);
+          int ch = lane & 7;
+          u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4));
+          if ((m >> 4) & 1) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
+          return v;
+        };
+        if (sums) {
+          // the sums themselves, rounded, before anything is applied to them
+          stage();
+#pragma unroll
+          for (int it = 0; it < 8; it++) {
+            if (it >= 4 * strips) continue;
+            const u32x4 v = staged(it);
+            int gm, gn;
+            const int64_t at = place(it, gm, gn);
+            if (gm < m_valid && gn < n_valid) *reinterpret_cast<u32x4*>(sums + at) = v;
+          }
+        }
         // (the activation of this pass's sums: arithmetic for the loads above to hide behind)
         if (activation != kNoActivation) {
 #pragma unroll
@@ -756,27 +796,11 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
             for (int j = 0; j < 2; j++)
               if (2 * qi + i < Cfg::IM) activate_all(acc[2 * qi + i][2 * qj + j], activation);
         }
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-          for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-              if (i >= strips) continue;
-              const f32x16_t& c = acc[(2 * qi + i) < Cfg::IM ? 2 * qi + i : 0][2 * qj + j];
-              int m = i * 32 + (lane & 31);
-              int ch = 4 * j + g;
-              u32x2 v = {pack2<Cfg::BF16>(c[4 * g], c[4 * g + 1]), pack2<Cfg::BF16>(c[4 * g + 2], c[4 * g + 3])};
-              *reinterpret_cast<u32x2*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4) + ((((lane >> 5) ^ (m >> 4)) & 1) << 3)) = v;
-            }
-        // no barrier: the staging buffer is private to the wavefront and LDS serves a wavefront's accesses in order
+        stage();
 #pragma unroll
         for (int it = 0; it < 8; it++) {
           if (it >= 4 * strips) continue;
-          int m = it * 8 + (lane >> 3);
-          int ch = lane & 7;
-          u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4));
-          if ((m >> 4) & 1) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
+          u32x4 v = staged(it);
           int gm, gn;
           int64_t at = place(it, gm, gn);
           bool wanted = gm < m_valid && gn < n_valid;
@@ -823,8 +847,16 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
     for (int slot = 0; slot < 3; slot++)
 #pragma unroll
       for (int r = 0; r < 16; r++) sum[r] += red[((wave * 3 + slot) * 16 + r) * 64 + lane];
-    if (activation != kNoActivation) activate_all(sum, activation);
     int gm = qi * 32 + (lane & 31);
+    if (sums) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        int gn = qj * 32 + 8 * g + 4 * (lane >> 5);
+        u32x2 v = {pack2<Cfg::BF16>(sum[4 * g], sum[4 * g + 1]), pack2<Cfg::BF16>(sum[4 * g + 2], sum[4 * g + 3])};
+        if (gm < m_valid && gn < n_valid) *reinterpret_cast<u32x2*>(sums + (int64_t)gm * ldc + gn) = v;
+      }
+    }
+    if (activation != kNoActivation) activate_all(sum, activation);
 #pragma unroll
     for (int g = 0; g < 4; g++) {
       int gn = qj * 32 + 8 * g + 4 * (lane >> 5);

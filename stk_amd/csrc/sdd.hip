@@ -64,7 +64,8 @@ __device__ __forceinline__ void sdd_tile64(const SddArgs& g, int r0, int p0, int
   const int block = have ? p0 + i * nseg + j : 0;
   const int n_valid = !have ? 0 : (cols - j < kWide ? cols - j : kWide) * 64;
   epilogue<Cfg, false>(acc, g.out + (int64_t)block * 4096, 64, have ? 64 : 0, n_valid, smem, 4096, g.activation,
-                       g.multiplier ? g.multiplier + (int64_t)block * 4096 : nullptr);
+                       g.multiplier ? g.multiplier + (int64_t)block * 4096 : nullptr, 0, 0, nullptr, nullptr, 0,
+                       g.sums ? g.sums + (int64_t)block * 4096 : nullptr);
 }
 
 template <class Quad, class Pair>
@@ -218,7 +219,20 @@ extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_
                              const int32_t* block_order, int64_t nnz,
                              int blocking, int dtype, int index_dtype, const uint8_t* plan,
                              int activation, const void* multiplier, stk_stream_t stream) {
+  return stk_sdd_fused_sums(lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, offsets, row_indices, column_indices,
+                            block_order, nnz, blocking, dtype, index_dtype, plan, activation, multiplier, nullptr, stream);
+}
+
+extern "C" int stk_sdd_fused_sums(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
+                                  const void* rhs, int64_t rhs_stride_k, int64_t rhs_stride_n,
+                                  int64_t m, int64_t k, int64_t n,
+                                  void* out, const int32_t* offsets, const void* row_indices, const void* column_indices,
+                                  const int32_t* block_order, int64_t nnz,
+                                  int blocking, int dtype, int index_dtype, const uint8_t* plan,
+                                  int activation, const void* multiplier, void* sums, stk_stream_t stream) {
   using namespace stk;
+  if (sums && (dtype == STK_F32 || !aligned16(sums) || sums == out))
+    return fail(STK_ERR_UNSUPPORTED, "stk_sdd_fused_sums: the sums go to a 16-byte aligned array of their own, 16-bit values only");
   if (dtype == STK_F32)
     return sdd_f32(lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, row_indices, column_indices, nnz, blocking,
                    index_dtype, activation, multiplier, static_cast<hipStream_t>(stream));
@@ -226,6 +240,7 @@ extern "C" int stk_sdd_fused(const void* lhs, int64_t lhs_stride_m, int64_t lhs_
   const int rc = sdd_problem("stk_sdd", lhs, lhs_stride_m, lhs_stride_k, rhs, rhs_stride_k, rhs_stride_n, m, k, n, out, offsets, row_indices,
                              column_indices, block_order, nnz, blocking, dtype, index_dtype, plan, activation, multiplier, &problem);
   if (rc != STK_OK || problem.empty) return rc;
+  problem.g.sums = static_cast<elem_t*>(sums);
   const SddArgs& g = problem.g;
   const bool ak = problem.ak, bk = problem.bk, stream_rhs = problem.stream_rhs;
   hipStream_t s = static_cast<hipStream_t>(stream);

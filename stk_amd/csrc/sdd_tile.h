@@ -28,6 +28,7 @@ struct SddArgs {
   const int32_t* row_slots;
   int top_k;
   int slots;
+  elem_t* sums;  // laid out like `out`: receives the rounded sums themselves (before activation and multiplier); or null
 };
 
 // The row of SddArgs::lhs that row `r` of a gathered lhs is taken from; negative: a row of zeros.
@@ -91,12 +92,12 @@ __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], co
     // Addressed as rows of the first block that run on, with the distance between the blocks added per block.
     const int64_t at = (int64_t)p[0][0] * BLK * BLK + (int64_t)m0 * BLK + n0;
     epilogue<Cfg, false>(acc, g.out + at, BLK, Cfg::TM - m0, BLK - n0, smem, 64, g.activation, g.multiplier ? g.multiplier + at : nullptr,
-                         m0, (int64_t)(p[1][0] - p[0][0] - 1) * BLK * BLK);
+                         m0, (int64_t)(p[1][0] - p[0][0] - 1) * BLK * BLK, nullptr, nullptr, 0, g.sums ? g.sums + at : nullptr);
   } else {
     const int block = p[m0 / BLK][n0 / BLK];  // the output block this wavefront writes into
     const int64_t at = (int64_t)(block < 0 ? 0 : block) * BLK * BLK + (int64_t)(m0 % BLK) * BLK + (n0 % BLK);
     epilogue<Cfg, false>(acc, g.out + at, BLK, block < 0 ? 0 : BLK - (m0 % BLK), BLK - (n0 % BLK), smem, 64, g.activation,
-                         g.multiplier ? g.multiplier + at : nullptr);
+                         g.multiplier ? g.multiplier + at : nullptr, 0, 0, nullptr, nullptr, 0, g.sums ? g.sums + at : nullptr);
   }
 }
 

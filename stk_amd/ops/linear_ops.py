@@ -34,12 +34,14 @@ def sdd(a, b, topo):
                   topo.column_indices_t, topo.offsets_t, topo.block_offsets_t)
 
 
-def sdd_fused(a, b, topo, activation=None, multiplier=None):
+def sdd_fused(a, b, topo, activation=None, multiplier=None, save_sums=False):
     """activation(sdd(a, b, topo)) * multiplier in one pass: the activation ("relu", "gelu_tanh",
     "gelu", "silu" or None) is applied to the fp32 sums before they are rounded, and the rounded
     values are multiplied by those of `multiplier` (a Matrix with topo's topology, or None) as
-    stk.ops.mul would (stk/ops/eltwise_ops.py:3-28).  Only the result is stored: the backward pass
-    computes the sums again (one more sdd) instead of keeping them."""
+    stk.ops.mul would (stk/ops/eltwise_ops.py:3-28).  By default only the result is stored and the
+    backward pass computes the sums again (one more sdd); with save_sums the product also stores the
+    rounded sums (one more array of values, what a caller of the reference keeps anyway) and the
+    backward pass is an element-wise pass over them."""
     assert isinstance(a, torch.Tensor)
     assert isinstance(b, torch.Tensor)
     assert isinstance(topo, Matrix)
@@ -47,6 +49,6 @@ def sdd_fused(a, b, topo, activation=None, multiplier=None):
     if multiplier is not None:
         assert isinstance(multiplier, Matrix)
         assert multiplier.size() == topo.size()
-    out = sputnik.sdd_fused(a, b, *_unpack(topo), activation, None if multiplier is None else multiplier.data)
+    out = sputnik.sdd_fused(a, b, *_unpack(topo), activation, None if multiplier is None else multiplier.data, save_sums)
     return Matrix(topo.size(), out, topo.row_indices, topo.column_indices, topo.offsets,
                   topo.column_indices_t, topo.offsets_t, topo.block_offsets_t)

@@ -199,8 +199,10 @@ def test_sdd_fused_dmoe_gated_layer():
 
 @pytest.mark.parametrize("activation,with_multiplier", [("gelu_tanh", False), ("silu", True), (None, True), ("relu", False), ("gelu", True)])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (True, True)])
-def test_sdd_fused_gradients(activation, with_multiplier, trans_a, trans_b):
-    # backward recomputes the sums; checked against torch autograd on the dense fp32 product gathered to blocks
+@pytest.mark.parametrize("save_sums", (False, True))
+def test_sdd_fused_gradients(activation, with_multiplier, trans_a, trans_b, save_sums):
+    # backward recomputes the sums, or reads the kept ones; checked against torch autograd on the dense fp32 product
+    # gathered to blocks, under the north-star tolerance and the two scale-free bounds
     _seed("sdd_fused_grad", activation, with_multiplier, trans_a, trans_b)
     m, k, n, b, dtype = 512, 128, 768, 128, torch.bfloat16
     a = _dense(*((k, m) if trans_a else (m, k)), dtype, std=0.3)
@@ -213,7 +215,7 @@ def test_sdd_fused_gradients(activation, with_multiplier, trans_a, trans_b):
         mult = stk.Matrix(topo_m.size(), values, topo_m.row_indices, topo_m.column_indices, topo_m.offsets,
                           topo_m.column_indices_t, topo_m.offsets_t, topo_m.block_offsets_t)
     weight = (torch.randn(topo_m.data.shape) * 0.1).to(dtype).to(DEV)
-    out = stk.ops.sdd_fused(lhs, rhs, topo_m, activation=activation, multiplier=mult)
+    out = stk.ops.sdd_fused(lhs, rhs, topo_m, activation=activation, multiplier=mult, save_sums=save_sums)
     (out.data.float() * weight.float()).sum().backward()
 
     lf, rf = lhs.detach().float().requires_grad_(True), rhs.detach().float().requires_grad_(True)
@@ -229,6 +231,34 @@ def test_sdd_fused_gradients(activation, with_multiplier, trans_a, trans_b):
     U.assert_close(bb.grad, U.np32(rf.grad.t() if trans_b else rf.grad), dtype, "fused grad wrt rhs")
     if with_multiplier:
         U.assert_close(mult.data.grad, U.np32(mf.grad), dtype, "fused grad wrt multiplier")
+        assert mult.data.grad.dtype == dtype
+        U.assert_close_scaled(mult.data.grad, mf.grad, dtype, "fused grad wrt multiplier")
+    U.assert_close_scaled(a.grad, lf.grad.t() if trans_a else lf.grad, dtype, "fused grad wrt lhs")
+    U.assert_close_scaled(bb.grad, rf.grad.t() if trans_b else rf.grad, dtype, "fused grad wrt rhs")
+
+
+@pytest.mark.parametrize("blocking,dtype", [(128, torch.bfloat16), (128, torch.float16), (64, torch.float16), (64, torch.bfloat16)])
+@pytest.mark.parametrize("m,k,n,sparsity", [(384, 128, 512, 0.5), (2048, 256, 2048, 0.7), (256, 96, 256, 0.0)])
+def test_sdd_fused_keeps_the_sums(m, k, n, sparsity, blocking, dtype):
+    # the second output of stk_sdd_fused_sums is the plain sdd, bit for bit, and the first is unchanged by it; the
+    # element-wise pass over the kept sums is within the tolerance of the product that applies the derivative itself
+    _seed("sdd_fused_sums", m, k, n, blocking, dtype)
+    lhs, rhs, topo_m, g = _fused_case(m, k, n, sparsity, blocking, dtype)
+    from stk_amd.backend import hip_kernels
+    meta = (topo_m.offsets, topo_m.row_indices, topo_m.column_indices)
+    plain, fused = torch.empty_like(topo_m.data), torch.empty_like(topo_m.data)
+    hip_kernels.sdd(lhs, rhs, tuple(topo_m.size()), plain, *meta)
+    hip_kernels.sdd_fused(lhs, rhs, tuple(topo_m.size()), fused, *meta, "gelu_tanh", g.data)
+    out, sums = torch.full_like(plain, float("nan")), torch.full_like(plain, float("nan"))
+    hip_kernels.sdd_fused(lhs, rhs, tuple(topo_m.size()), out, *meta, "gelu_tanh", g.data, sums=sums)
+    assert torch.equal(sums.view(torch.int16), plain.view(torch.int16))
+    assert torch.equal(out.view(torch.int16), fused.view(torch.int16))
+    for kind in ("gelu_tanh_grad", "silu_grad", "relu_grad", "gelu_grad", "relu", "gelu"):
+        # (on the kept, rounded sums: where an activation bends, its derivative at a rounded sum is not within the
+        # tolerance of its derivative at the fp32 sum, which is what the product that recomputes the sums uses)
+        want = O.activation(U.np32(sums).astype(np.float64), kind) * U.np32(g.data).astype(np.float64)
+        U.assert_close(hip_kernels.activation_product(sums, g.data, kind), want, dtype, kind)
+    assert torch.equal(hip_kernels.activation_product(sums, None, None), sums)
 
 
 @pytest.mark.parametrize("blocking,dtype", [(128, torch.bfloat16), (64, torch.float16)])
