@@ -149,8 +149,9 @@ int stk_sdd(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride_k,
  * act (an STK_ACT_* code) is applied to the fp32 sums, the result is rounded to `dtype`;
  * multiplier, if not NULL, holds the values [nnz, b, b] of a matrix with the same topology
  * (16-byte aligned, same dtype, may be `out` itself only if no other stream reads it), and the
- * product of the two 16-bit values is rounded once more - what an activation on the values of the
- * sparse result followed by mul(), stk/ops/eltwise_ops.py:3-28, gives (the reference and its callers
+ * product of the two 16-bit values is rounded once more (with one of the derivative codes, whose product with the
+ * multiplier is a gradient, the fp32 derivative is multiplied and the product rounded once) - what an activation on the
+ * values of the sparse result followed by mul(), stk/ops/eltwise_ops.py:3-28, gives (the reference and its callers
  * run these as separate passes over the values: MoE layers apply the activation to the result of
  * sdd(), stk/ops/linear_ops.py:37-59, and gated layers multiply two such results).  With
  * STK_ACT_NONE and no multiplier it is stk_sdd.  All other arguments as for stk_sdd.
@@ -180,8 +181,9 @@ int stk_sdd_fused_sums(const void* lhs, int64_t lhs_stride_m, int64_t lhs_stride
                        int activation, const void* multiplier, void* sums, stk_stream_t stream);
 
 /*
- * out[i] = round(round(act(sums[i])) * factor[i]) for i < count (factor NULL: the first rounding only): the
- * element-wise arithmetic of stk_sdd_fused's store applied to stored 16-bit sums.  act is any STK_ACT_* code; with a
+ * out[i] = round(round(act(sums[i])) * factor[i]) for i < count (factor NULL: the first rounding only; a derivative
+ * code: round(act'(sums[i]) * factor[i]), one rounding): the element-wise arithmetic of stk_sdd_fused's store applied
+ * to stored 16-bit sums.  act is any STK_ACT_* code; with a
  * derivative and the incoming gradient as `factor` this is the gradient with respect to the sums.  count a multiple
  * of 8, arrays 16-byte aligned, `out` may be `factor` or `sums`.  Stands in for the element-wise passes that the
  * reference's callers run in torch on the values of a Matrix (stk/ops/eltwise_ops.py:3-28 is their multiplication).

@@ -583,6 +583,9 @@ NNZ_POLL_LIMIT = 200000   # polls of the pinned nnz word (some 20 ms) before to_
 _nnz_buffers = threading.local()   # per host thread: device index -> pinned int32[1] that stk_to_sparse_count_nnz writes nnz into
 
 
+_TO_SPARSE_KEEP_BYTES = 1 << 16   # scratch allocations below this size stay alive behind the views returned
+
+
 def to_sparse(x, blocking, index_dtype=torch.int16):
     """(data, row_indices, column_indices, offsets) of the nonzero blocks of x."""
     _need_gpu(x)
@@ -633,6 +636,13 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
         _lib.check(lib.stk_to_sparse_gather(
             x.data_ptr(), rows, cols, x.stride(0), blocking, _elem_bytes(x), row_indices.data_ptr(), column_indices.data_ptr(), nnz,
             _INDEX_DTYPES[index_dtype], data.data_ptr(), _stream()))
+        # A Matrix keeps these tensors for as long as it lives.  Where the room for every block is much more than the
+        # nonzero blocks need (a large, very sparse matrix), they are copied out of it, and the offsets out of the
+        # allocation they share with the block mask, so that the O(rows x columns / blocking^2) buffers can go.
+        if room.numel() * room.element_size() >= _TO_SPARSE_KEEP_BYTES and 4 * nnz <= br * bc:
+            row_indices, column_indices = row_indices.clone(), column_indices.clone()
+        if scratch.numel() >= _TO_SPARSE_KEEP_BYTES and 4 * 4 * (br + 1) <= scratch.numel():
+            offsets = offsets.clone()
     return data, row_indices, column_indices, offsets
 
 

@@ -13,6 +13,9 @@
 #define STK_SDD_KT 32
 #define STK_SDD_STAGES 4
 #endif
+#ifndef STK_SDD_PERSISTENT
+#define STK_SDD_PERSISTENT 1   // stk_sdd with a plan: one workgroup per compute unit that walks the tile list
+#endif
 #ifndef STK_DSD_KT
 #define STK_DSD_KT 32
 #define STK_DSD_STAGES 4
@@ -155,6 +158,13 @@ inline void set_lds_limit(Kernel kernel, int bytes) {
 // Read-only metadata read through the constant address space: wave-uniform loads become scalar loads.
 typedef const __attribute__((address_space(4))) int32_t* cint_t;
 __device__ __forceinline__ cint_t const_ints(const void* p) { return (cint_t)(uintptr_t)p; }
+
+// Entry i of an index array through the scalar unit (a wave-uniform i; 16-bit entries are read as halves of 32-bit
+// words, so the array must start at a multiple of four bytes).
+__device__ __forceinline__ int scalar_index(const void* p, int i, int idx32) {
+  if (idx32) return const_ints(p)[i];
+  return (int)(int16_t)(const_ints(p)[i >> 1] >> (16 * (i & 1)));
+}
 
 __device__ __forceinline__ int load_index(const void* __restrict__ p, int64_t i, int idx32) {
   return idx32 ? static_cast<const int32_t*>(p)[i] : static_cast<int>(static_cast<const int16_t*>(p)[i]);

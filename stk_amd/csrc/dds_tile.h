@@ -73,10 +73,6 @@ __device__ __forceinline__ DdsWalk<LINES> dds_walk(const DdsArgs& g, int bj, int
 // transfers of the current one are in flight without touching their in-order completion count.  False (and w
 // incomplete) when the walk is longer or the index arrays cannot be read as 32-bit words.
 constexpr int kScalarWalk = 4;
-__device__ __forceinline__ int scalar_index(const void* p, int i, int idx32) {
-  if (idx32) return const_ints(p)[i];
-  return (int)(int16_t)(const_ints(p)[i >> 1] >> (16 * (i & 1)));
-}
 template <int LINES, bool TRANS_B>
 __device__ __forceinline__ bool dds_walk_scalar(const DdsArgs& g, int bj, int lines, DdsWalk<LINES>& w) {
   w.bj = bj;

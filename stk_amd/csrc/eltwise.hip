@@ -2,7 +2,7 @@
 // element - the step of a backward pass that stk_sdd_fused_sums makes possible: with the sums of the forward product
 // kept, the gradient with respect to them is act'(sums) * incoming gradient, one pass over the values instead of a
 // product that computes the sums again.  Same arithmetic as the store of stk_sdd_fused: the function in fp32, rounded,
-// then the product of the two 16-bit values rounded once more.
+// then the product of the two 16-bit values rounded once more; a derivative times its factor is rounded once.
 #include "common.h"
 #include "gemm_core.h"
 
@@ -36,8 +36,14 @@ __global__ __launch_bounds__(256) void activation_product_kernel(const u32x4* __
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const f32x2_t x = unpack2<BF16>(v[j]);
-      v[j] = pack2<BF16>(activate_one(x.x, activation), activate_one(x.y, activation));
-      if (factor) v[j] = mul_packed<BF16>(v[j], fs[j]);
+      const float lo = activate_one(x.x, activation), hi = activate_one(x.y, activation);
+      if (factor && activation >= kReluGrad) {
+        const f32x2_t y = unpack2<BF16>(fs[j]);
+        v[j] = pack2<BF16>(lo * y.x, hi * y.y);
+      } else {
+        v[j] = pack2<BF16>(lo, hi);
+        if (factor) v[j] = mul_packed<BF16>(v[j], fs[j]);
+      }
     }
     __builtin_nontemporal_store(u32x4{v[0], v[1], v[2], v[3]}, out + i);
   }

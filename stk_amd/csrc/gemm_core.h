@@ -692,7 +692,9 @@ __device__ __forceinline__ void mainloop_reg(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
 // the sub-tile's first), for outputs made of 128-row blocks that do not follow each other in memory.
 // activation (wave-uniform): applied to the fp32 sums before they are rounded.
 // mul (wave-uniform, or null): an array laid out like `out`, pointing at the same element; the rounded
-// values are multiplied by its elements and rounded again.
+// values are multiplied by its elements and rounded again.  With the derivative of an activation the product is a
+// gradient, not the product of two stored matrices: the fp32 derivative is multiplied by the element and the product
+// is rounded once.
 // SCATTER: row gm of the sub-tile goes to row row_map[gm] of the array whose row 0 `out` then points into (at the
 // sub-tile's first column); rows whose entry is negative or not below out_rows are dropped.  row_scale (or null):
 // fp32 factors by destination row; the rounded values are multiplied by them and rounded again.
@@ -740,8 +742,9 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
           for (int it = 0; it < 8; it++) scale[it] = (row_scale && dest[it] >= 0) ? row_scale[dest[it]] : 1.0f;
         }
         // the multiplier's values of this pass, read once: on their way while the sums are rounded and staged
+        const bool one_rounding = mul && activation >= kReluGrad;
         u32x4 factor[8];
-        if (mul) {
+        if (mul && !one_rounding) {
 #pragma unroll
           for (int it = 0; it < 8; it++) {
             int gm, gn;
@@ -796,6 +799,34 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
             for (int j = 0; j < 2; j++)
               if (2 * qi + i < Cfg::IM) activate_all(acc[2 * qi + i][2 * qj + j], activation);
         }
+        if (one_rounding) {
+          // the multiplier's elements where the accumulators hold theirs: lane l has row 32 i + l % 32 and the four
+          // columns from 32 j + 8 g + 4 (l / 32) of this pass's quadrant in values 4 g .. 4 g + 3
+          u32x2 f[2][2][4];
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+              for (int g = 0; g < 4; g++) {
+                const int gm = qi * 64 + i * 32 + (lane & 31), n = j * 32 + 8 * g + 4 * (lane >> 5);
+                f[i][j][g] = u32x2{0u, 0u};
+                if (i < strips && gm < m_valid && qj * 64 + n < n_valid)
+                  f[i][j][g] = *reinterpret_cast<const u32x2*>(mul + (int64_t)gm * ldc + qj * quadrant_stride + n +
+                                                               (int64_t)((row_base + gm) >> 7) * row_jump);
+              }
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+              for (int g = 0; g < 4; g++) {
+                if (i >= strips) continue;
+                f32x16_t& c = acc[(2 * qi + i) < Cfg::IM ? 2 * qi + i : 0][2 * qj + j];
+                const f32x2_t lo = unpack2<Cfg::BF16>(f[i][j][g].x), hi = unpack2<Cfg::BF16>(f[i][j][g].y);
+                c[4 * g] *= lo.x, c[4 * g + 1] *= lo.y, c[4 * g + 2] *= hi.x, c[4 * g + 3] *= hi.y;
+              }
+        }
         stage();
 #pragma unroll
         for (int it = 0; it < 8; it++) {
@@ -809,7 +840,7 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
             at = (int64_t)dest[it] * ldc + gn;
           }
           if (wanted) {
-            if (mul) {
+            if (mul && !one_rounding) {
               const u32x4 f = factor[it];
               v = u32x4{mul_packed<Cfg::BF16>(v.x, f.x), mul_packed<Cfg::BF16>(v.y, f.y), mul_packed<Cfg::BF16>(v.z, f.z), mul_packed<Cfg::BF16>(v.w, f.w)};
             }
@@ -864,7 +895,12 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
       if (gm < m_valid && gn < n_valid) {
         if (mul) {
           const u32x2 f = *reinterpret_cast<const u32x2*>(mul + (int64_t)gm * ldc + gn);
-          v = u32x2{mul_packed<Cfg::BF16>(v.x, f.x), mul_packed<Cfg::BF16>(v.y, f.y)};
+          if (activation >= kReluGrad) {
+            const f32x2_t lo = unpack2<Cfg::BF16>(f.x), hi = unpack2<Cfg::BF16>(f.y);
+            v = u32x2{pack2<Cfg::BF16>(sum[4 * g] * lo.x, sum[4 * g + 1] * lo.y), pack2<Cfg::BF16>(sum[4 * g + 2] * hi.x, sum[4 * g + 3] * hi.y)};
+          } else {
+            v = u32x2{mul_packed<Cfg::BF16>(v.x, f.x), mul_packed<Cfg::BF16>(v.y, f.y)};
+          }
         }
         *reinterpret_cast<u32x2*>(out + (int64_t)gm * ldc + gn) = v;
       }

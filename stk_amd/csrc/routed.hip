@@ -41,7 +41,10 @@ static void launch_gather128(const SddArgs& g, hipStream_t stream) {
   constexpr int lds = lds0 > Triple::kSmemBytes ? lds0 : Triple::kSmemBytes;
   static const int once = (set_lds_limit(&sdd_gather_fused_kernel<Quad, Pair, Triple>, lds), 0);
   (void)once;
-  const int grid = g.tiles ? (int)sdd_max_tiles(g.block_rows, g.nnz) : (g.nnz + 1) / 2;
+  // with a plan: one workgroup per compute unit (the tiles' LDS leaves room for one), which walks the list of tiles;
+  // at most one tile per two blocks of a row, rounded up per row
+  const int most = (int)sdd_max_tiles(g.block_rows, g.nnz), units = STK_SDD_PERSISTENT ? compute_units() : 0;
+  const int grid = g.tiles ? (units > 0 && units < most ? units : most) : (g.nnz + 1) / 2;
   hipLaunchKernelGGL((sdd_gather_fused_kernel<Quad, Pair, Triple>), dim3(grid), dim3(512), lds, stream, g);
 }
 

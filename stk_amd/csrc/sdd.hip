@@ -115,7 +115,10 @@ static void launch_sdd128(const SddArgs& g, hipStream_t stream) {
   static const int once = (set_lds_limit(&sdd_fused_kernel<Quad, Pair, Triple, true>, lds), 0);
   (void)once;
   // with a plan: at most one tile per two blocks of a row, rounded up per row
-  const int grid = g.tiles ? (int)sdd_max_tiles(g.block_rows, g.nnz) : (g.nnz + 1) / 2;
+  // with a plan: one workgroup per compute unit (the tiles' LDS leaves room for one), which walks the list of tiles;
+  // at most one tile per two blocks of a row, rounded up per row
+  const int most = (int)sdd_max_tiles(g.block_rows, g.nnz), units = STK_SDD_PERSISTENT ? compute_units() : 0;
+  const int grid = g.tiles ? (units > 0 && units < most ? units : most) : (g.nnz + 1) / 2;
   hipLaunchKernelGGL((sdd_fused_kernel<Quad, Pair, Triple, true>), dim3(grid), dim3(512), lds, stream, g);
 }
 
@@ -203,6 +206,7 @@ int stk::sdd_problem(const char* who, const void* lhs, int64_t lhs_stride_m, int
                  static_cast<elem_t*>(out), offsets, row_indices, column_indices, block_order,
                  plan && offsets ? reinterpret_cast<const int32_t*>(plan) : nullptr, (int)nnz, (int)(m / blocking), index_dtype == STK_I32,
                  activation, static_cast<const elem_t*>(multiplier)};
+  p->g.scalar_indices = index_dtype == STK_I32 || !((reinterpret_cast<uintptr_t>(row_indices) | reinterpret_cast<uintptr_t>(column_indices)) & 3u);
   p->ak = ak;
   p->bk = bk;
   // an rhs column panel is read once per tile that holds a block of that block column: with few

@@ -29,6 +29,7 @@ struct SddArgs {
   int top_k;
   int slots;
   elem_t* sums;  // laid out like `out`: receives the rounded sums themselves (before activation and multiplier); or null
+  int scalar_indices;  // row_indices and column_indices may be read through the scalar unit (see scalar_index())
 };
 
 // The row of SddArgs::lhs that row `r` of a gathered lhs is taken from; negative: a row of zeros.
@@ -41,8 +42,10 @@ __device__ __forceinline__ int gathered_row(const SddArgs& g, int r) {
 // block rows / columns, p[i][j] the output block ids (negative: not stored).
 // GATHER: the rows of the lhs are gathered (SddArgs::row_slots); the transfers of the lhs tiles then take every row
 // from where it lies, and rows of zeros are computed on the array's first row and set to zero afterwards.
-template <class Cfg, int BLK, bool FULL, bool GATHER = false>
-__device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem) {
+// after_prologue: see mainloop_dma (direct-to-LDS pipeline only).
+template <class Cfg, int BLK, bool FULL, bool GATHER = false, class Hook>
+__device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem,
+                                         Hook&& after_prologue) {
   static_assert(Cfg::PM == BLK && Cfg::PN == BLK && Cfg::A_PARTS <= 3 && Cfg::B_PARTS <= 2, "one operand part per block row / column");
   static_assert(!GATHER || (FULL && Cfg::A_KMAJOR), "gathered rows: row-major lhs, direct-to-LDS pipeline");
   constexpr int KT = Cfg::KT;
@@ -63,12 +66,12 @@ __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], co
     return TilePtrs{{a0[0] + t * a_step, a0[1] + t * a_step, a0[2] + t * a_step}, {b0[0] + t * b_step, b0[1] + t * b_step}, left < KT ? left : KT};
   };
   if constexpr (GATHER) {
-    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem, [] {}, [&](int q, int row) {
+    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem, after_prologue, [&](int q, int row) {
       const int from = gathered_row(g, r[q] * BLK + row);
       return from < 0 ? 0 : from;
     });
   } else if constexpr (FULL) {
-    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem);
+    mainloop_dma<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, smem, after_prologue);
   } else {
     mainloop_reg<Cfg>(acc, ntiles, tile_fn, g.lda, g.ldb, BLK, BLK, smem);
   }
@@ -101,29 +104,60 @@ __device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], co
   }
 }
 
+template <class Cfg, int BLK, bool FULL, bool GATHER = false>
+__device__ __forceinline__ void sdd_tile(const SddArgs& g, const int (&r)[3], const int (&c)[2], const int (&p)[3][2], char* smem) {
+  sdd_tile<Cfg, BLK, FULL, GATHER>(g, r, c, p, smem, [] {});
+}
+
+// A tile of the plan's list (128-blocks): its first block, its shape (rows | columns << 8), the block row and the
+// number of blocks in it, and the block columns of its one or two blocks.
+struct SddPlanTile {
+  int p0, shape, r0, nseg, c0, c1;
+};
+// SCALAR: through the scalar unit only (SddArgs::scalar_indices must hold): nothing that counts as a vector memory
+// operation, so that it can run while the transfers of a tile are in flight.
+template <bool SCALAR>
+__device__ __forceinline__ SddPlanTile sdd_plan_tile_of(const SddArgs& g, int item) {
+  SddPlanTile t;
+  t.p0 = const_ints(g.tiles)[2 + 2 * item], t.shape = const_ints(g.tiles)[3 + 2 * item];
+  const bool has1 = (t.shape >> 8) == 2;
+  if constexpr (SCALAR) {
+    t.r0 = scalar_index(g.row_indices, t.p0, g.idx32);
+    t.c0 = scalar_index(g.column_indices, t.p0, g.idx32);
+    t.c1 = has1 ? scalar_index(g.column_indices, t.p0 + 1, g.idx32) : t.c0;
+  } else {
+    t.r0 = uniform(load_index(g.row_indices, t.p0, g.idx32));
+    t.c0 = uniform(load_index(g.column_indices, t.p0, g.idx32));
+    t.c1 = has1 ? uniform(load_index(g.column_indices, t.p0 + 1, g.idx32)) : t.c0;
+  }
+  t.nseg = const_ints(g.offsets)[t.r0 + 1] - const_ints(g.offsets)[t.r0];
+  return t;
+}
+
 // The tile `item` of the plan's list (128-blocks): two neighbouring blocks of a block row (1x2 blocks, 128x256),
 // together with the two blocks below when the next row repeats this one (2x2 blocks, 256x256), or one block with
 // the two below it for the last three rows of a run of odd length (3x1 blocks, 384x128).
-template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
-__device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* smem) {
-  const int p0 = const_ints(g.tiles)[2 + 2 * item], shape = const_ints(g.tiles)[3 + 2 * item];
-  const int r0 = uniform(load_index(g.row_indices, p0, g.idx32));
-  const bool has1 = (shape >> 8) == 2;  // an odd row ends with a tile of one block
-  const int rows = shape & 0xff, nseg = const_ints(g.offsets)[r0 + 1] - const_ints(g.offsets)[r0];
+template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false, class Hook>
+__device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, const SddPlanTile& t, char* smem, Hook&& after_prologue) {
+  const int p0 = t.p0, r0 = t.r0, nseg = t.nseg, c0 = t.c0, c1 = t.c1;
+  const bool has1 = (t.shape >> 8) == 2;  // an odd row ends with a tile of one block
+  const int rows = t.shape & 0xff;
   const int below = rows >= 2 ? p0 + nseg : -1;
-  const int c0 = uniform(load_index(g.column_indices, p0, g.idx32));
-  const int c1 = has1 ? uniform(load_index(g.column_indices, p0 + 1, g.idx32)) : c0;
   if (rows == 3) {
     // the last three rows of a run of identical rows: one block wide, so that the rhs panel is read once for the three
     const int rr[3] = {r0, r0 + 1, r0 + 2}, cc[2] = {c0, c0}, pp[3][2] = {{p0, -1}, {below, -1}, {below + nseg, -1}};
-    sdd_tile<Triple, 128, FULL, GATHER>(g, rr, cc, pp, smem);
+    sdd_tile<Triple, 128, FULL, GATHER>(g, rr, cc, pp, smem, after_prologue);
   } else if (below >= 0) {
     const int rr[3] = {r0, r0 + 1, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {below, has1 ? below + 1 : -1}, {-1, -1}};
-    sdd_tile<Quad, 128, FULL, GATHER>(g, rr, cc, pp, smem);
+    sdd_tile<Quad, 128, FULL, GATHER>(g, rr, cc, pp, smem, after_prologue);
   } else {
     const int rr[3] = {r0, r0, r0}, cc[2] = {c0, c1}, pp[3][2] = {{p0, has1 ? p0 + 1 : -1}, {-1, -1}, {-1, -1}};
-    sdd_tile<Pair, 128, FULL, GATHER>(g, rr, cc, pp, smem);
+    sdd_tile<Pair, 128, FULL, GATHER>(g, rr, cc, pp, smem, after_prologue);
   }
+}
+template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
+__device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* smem) {
+  sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, sdd_plan_tile_of<false>(g, item), smem, [] {});
 }
 
 // What workgroup blockIdx.x of a launch over 128-blocks with eight wavefronts computes: its tile of the plan's list,
@@ -131,10 +165,29 @@ __device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* 
 template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void sdd_fused_tile(const SddArgs& g, char* smem) {
   if (g.tiles) {
+    // The launch has one workgroup per compute unit (or fewer tiles than that): every workgroup walks the list from
+    // its own id in steps of the grid, which leaves a tile on the compute die it would have run on as a workgroup
+    // of its own (the dies take workgroup ids in turn, and the step is a multiple of their number).
+    // While the first transfers of a tile are in flight, the next tile's entry of the list and its indices are looked
+    // up through the scalar unit.
     const int count = const_ints(g.tiles)[0];
     if ((int)blockIdx.x >= count) return;
-    const int item = xcd_tile(blockIdx.x, count);
-    sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, item, smem);
+    SddPlanTile tile = sdd_plan_tile_of<false>(g, xcd_tile(blockIdx.x, count));
+    for (int id = blockIdx.x; id < count; id += gridDim.x) {
+      const int next_id = id + gridDim.x;
+      SddPlanTile next = tile;
+      bool looked_up = false;
+      if constexpr (FULL) {
+        sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [&] {
+          if (next_id < count && g.scalar_indices) next = sdd_plan_tile_of<true>(g, xcd_tile(next_id, count)), looked_up = true;
+        });
+      } else {
+        sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [] {});
+      }
+      if (next_id < count && !looked_up) next = sdd_plan_tile_of<false>(g, xcd_tile(next_id, count));
+      tile = next;
+      __syncthreads();  // the epilogue staging buffer is part of the next tile's first stage
+    }
     return;
   }
   const int npairs = (g.nnz + 1) >> 1;

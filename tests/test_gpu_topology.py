@@ -440,3 +440,21 @@ def test_dmoe_topology_builder_rejects_bad_arguments():
         hip_kernels.dmoe_topology(bins, 128, 1, 0)
     with pytest.raises(AssertionError):                      # 40000 block columns do not fit 16-bit indices
         hip_kernels.dmoe_topology(bins, 128, 1, 40000)
+
+
+def test_to_sparse_of_a_large_sparse_matrix_keeps_only_what_it_uses():
+    # 1024 x 1024 blocks of 8 with 37 of them nonzero: the index tensors and the offsets own their storage, so that a
+    # Matrix does not hold on to the buffers sized for every block that the conversion works in
+    rows = cols = 8192
+    x = torch.zeros(rows, cols, dtype=torch.float16, device=DEV)
+    g = torch.Generator().manual_seed(4)
+    where = torch.randperm(1024 * 1024, generator=g)[:37]
+    for w in where.tolist():
+        x[(w // 1024) * 8 + 3, (w % 1024) * 8 + 5] = 1.0
+    m = stk.ops.to_sparse(x, 8)
+    assert m.row_indices.numel() == 37
+    for t, elems in ((m.row_indices, 37), (m.column_indices, 37), (m.offsets, 1025)):
+        assert t.untyped_storage().nbytes() <= max(512, 2 * elems * t.element_size()), t.untyped_storage().nbytes()
+    data, topo = O.to_sparse(x.cpu().numpy(), 8)
+    U.assert_topology_equal(m, topo, "large sparse")
+    assert torch.equal(stk.ops.to_dense(m), x)
