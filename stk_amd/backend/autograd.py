@@ -68,9 +68,14 @@ def _run_sdd(lhs, rhs, sp):
 # fill the compute units that the other leaves idle in its last round.
 OVERLAP_GRADIENTS = True
 _side_streams = {}
-# Both gradients of sdd (stk_dsd_dds, stk_dsd_dsd) and of dsd (stk_sdd_dsd) in one launch each where the operands' layouts allow it,
-# instead of two launches side by side; the same results.
+# Both gradients of sdd (stk_dsd_dds, stk_dsd_dsd) in one launch where the operands' layouts allow it, instead of two
+# launches side by side; the same results.
 JOINT_GRADIENTS = True
+# The same for both gradients of dsd (stk_sdd_dsd).  What a joint launch gains is its tail: the short tiles of the second
+# product fill the compute units that the last round of the first leaves idle.  An sdd that runs as one workgroup per
+# compute unit walking its tile list has no such round left, and the two launches are then the shorter way (benchmark
+# topology, sdd(dy, W2^T) + dsd(h^T, dy) back to back: 462 us as two launches, 473 us as one).
+JOINT_DSD_GRADIENTS = False
 
 
 def _side_stream(device):
@@ -121,7 +126,7 @@ class DSD(torch.autograd.Function):
         dy = _plain(dy)
         want_data = want_rhs = None
         rhs_is_view = _is_transposed_view(rhs)
-        if JOINT_GRADIENTS and dy.is_cuda and ctx.needs_input_grad[1] and ctx.needs_input_grad[9] and not rhs_is_view:
+        if JOINT_DSD_GRADIENTS and dy.is_cuda and ctx.needs_input_grad[1] and ctx.needs_input_grad[9] and not rhs_is_view:
             # dy rhs^T on the pattern and op(S)^T dy read the same dy: one call (sputnik.py:131-155 makes two)
             ddata = torch.empty_like(data)
             drhs = torch.empty_like(rhs, memory_format=torch.contiguous_format)

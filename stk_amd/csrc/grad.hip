@@ -98,18 +98,18 @@ static void launch_dsd_dsd(const DsdArgs& d, const PlanLists& rows, const DsdArg
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, d, rows, t, cols);
 }
 
-// 128-blocks, eight wavefronts: the tiles of the sdd from the plan's tile list as in sdd_fused_kernel, then the tiles
-// of the dsd from the plan's lists of lines as in dsd_fused_kernel.  The grid is an upper bound for both.
+// 128-blocks, eight wavefronts: the first `walkers` workgroups (one per compute unit) walk the tile list of the sdd as
+// in sdd_fused_kernel; the workgroups behind them take the tiles of the dsd from the plan's lists of lines as in
+// dsd_fused_kernel, one each, as the walkers leave.  The grid is an upper bound for the dsd.
 template <class SddQuad, class SddPair, class SddTriple, class DsdFused, class DsdTriple, class DsdSingle, bool TRANS_A>
-__global__ __launch_bounds__(512, 2) void sdd_dsd_kernel(SddArgs a, DsdArgs d, PlanLists lines) {
+__global__ __launch_bounds__(512, 2) void sdd_dsd_kernel(SddArgs a, DsdArgs d, PlanLists lines, int walkers) {
   extern __shared__ __align__(16) char smem[];
-  const int count = const_ints(a.tiles)[0];
   int bid = blockIdx.x;
-  if (bid < count) {
-    sdd_plan_tile<SddQuad, SddPair, SddTriple, true>(a, xcd_tile(bid, count), smem);
+  if (bid < walkers) {
+    sdd_walk_plan<SddQuad, SddPair, SddTriple, true>(a, bid, walkers, smem);
     return;
   }
-  bid -= count;
+  bid -= walkers;
   dsd_plan_tile<DsdFused, DsdTriple, DsdSingle, TRANS_A>(d, lines, bid, smem);
 }
 
@@ -130,9 +130,11 @@ static void launch_sdd_dsd(const SddArgs& a, const DsdArgs& d, const PlanLists& 
   auto kernel = &sdd_dsd_kernel<SddQuad, SddPair, SddTriple, DsdFused, DsdTriple, DsdSingle, TRANS_A>;
   static const int once = (set_lds_limit(kernel, lds), 0);
   (void)once;
-  // upper bound: the tile list of the sdd at its longest, every line of the dsd a tile of its own
-  const int grid = (int)sdd_max_tiles(a.block_rows, a.nnz) + d.block_rows * (d.n / DsdFused::TN);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, a, d, lines);
+  // the walkers of the sdd (as many as it would have workgroups on its own), then every line of the dsd a tile of its own
+  const int most = (int)sdd_max_tiles(a.block_rows, a.nnz), units = STK_SDD_PERSISTENT ? compute_units() : 0;
+  const int walkers = units > 0 && units < most ? units : most;
+  const int grid = walkers + d.block_rows * (d.n / DsdFused::TN);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, a, d, lines, walkers);
 }
 
 }  // namespace stk

@@ -160,34 +160,40 @@ __device__ __forceinline__ void sdd_plan_tile(const SddArgs& g, int item, char* 
   sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, sdd_plan_tile_of<false>(g, item), smem, [] {});
 }
 
-// What workgroup blockIdx.x of a launch over 128-blocks with eight wavefronts computes: its tile of the plan's list,
-// or without a plan the blockIdx.x-th pair of blocks in CSR order (every row on its own).
+// The tiles first, first + stride, ... of the plan's list, one after the other (a workgroup of a launch with fewer
+// workgroups than tiles: one per compute unit).  With a stride that is a multiple of the number of compute dies,
+// which take workgroup ids in turn, every tile stays on the die it would have run on as a workgroup of its own.
+// While the first transfers of a tile are in flight, the next tile's entry of the list and its indices are looked
+// up through the scalar unit.
+template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
+__device__ __forceinline__ void sdd_walk_plan(const SddArgs& g, int first, int stride, char* smem) {
+  const int count = const_ints(g.tiles)[0];
+  if (first >= count) return;
+  SddPlanTile tile = sdd_plan_tile_of<false>(g, xcd_tile(first, count));
+  for (int id = first; id < count; id += stride) {
+    const int next_id = id + stride;
+    SddPlanTile next = tile;
+    bool looked_up = false;
+    if constexpr (FULL) {
+      sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [&] {
+        if (next_id < count && g.scalar_indices) next = sdd_plan_tile_of<true>(g, xcd_tile(next_id, count)), looked_up = true;
+      });
+    } else {
+      sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [] {});
+    }
+    if (next_id < count && !looked_up) next = sdd_plan_tile_of<false>(g, xcd_tile(next_id, count));
+    tile = next;
+    __syncthreads();  // the epilogue staging buffer is part of the next tile's first stage
+  }
+}
+
+// What workgroup blockIdx.x of a launch over 128-blocks with eight wavefronts computes: its tiles of the plan's list
+// (the launch has one workgroup per compute unit, or fewer tiles than that), or without a plan the blockIdx.x-th pair
+// of blocks in CSR order (every row on its own).
 template <class Quad, class Pair, class Triple, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void sdd_fused_tile(const SddArgs& g, char* smem) {
   if (g.tiles) {
-    // The launch has one workgroup per compute unit (or fewer tiles than that): every workgroup walks the list from
-    // its own id in steps of the grid, which leaves a tile on the compute die it would have run on as a workgroup
-    // of its own (the dies take workgroup ids in turn, and the step is a multiple of their number).
-    // While the first transfers of a tile are in flight, the next tile's entry of the list and its indices are looked
-    // up through the scalar unit.
-    const int count = const_ints(g.tiles)[0];
-    if ((int)blockIdx.x >= count) return;
-    SddPlanTile tile = sdd_plan_tile_of<false>(g, xcd_tile(blockIdx.x, count));
-    for (int id = blockIdx.x; id < count; id += gridDim.x) {
-      const int next_id = id + gridDim.x;
-      SddPlanTile next = tile;
-      bool looked_up = false;
-      if constexpr (FULL) {
-        sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [&] {
-          if (next_id < count && g.scalar_indices) next = sdd_plan_tile_of<true>(g, xcd_tile(next_id, count)), looked_up = true;
-        });
-      } else {
-        sdd_plan_tile<Quad, Pair, Triple, FULL, GATHER>(g, tile, smem, [] {});
-      }
-      if (next_id < count && !looked_up) next = sdd_plan_tile_of<false>(g, xcd_tile(next_id, count));
-      tile = next;
-      __syncthreads();  // the epilogue staging buffer is part of the next tile's first stage
-    }
+    sdd_walk_plan<Quad, Pair, Triple, FULL, GATHER>(g, blockIdx.x, gridDim.x, smem);
     return;
   }
   const int npairs = (g.nnz + 1) >> 1;

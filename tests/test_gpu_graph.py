@@ -67,7 +67,10 @@ def test_forward_chain_replays_from_a_graph(blocking, dtype, warm_up_on_capture_
     U.assert_close(got[1], O.dsd(topo.shape, U.np32(got[0]), topo, False, U.np32(w2)), dtype, "dsd from the graph")
 
 
-def test_forward_and_backward_replay_from_a_graph():
+@pytest.mark.parametrize("joint_dsd_gradients", (False, True))
+def test_forward_and_backward_replay_from_a_graph(joint_dsd_gradients, monkeypatch):
+    from stk_amd.backend import autograd
+    monkeypatch.setattr(autograd, "JOINT_DSD_GRADIENTS", joint_dsd_gradients)
     dtype = torch.bfloat16
     topo, tm, x, w1, w2, g = _case(1024, 4096, 128, dtype, 43)
     xs, w1s, w2s = (t.detach().clone().requires_grad_(True) for t in (x, w1, w2))
@@ -78,7 +81,8 @@ def test_forward_and_backward_replay_from_a_graph():
 
     def forward():
         h = stk.ops.sdd(xs, w1s, tm)
-        # dsd's gradients are one launch, those of the dds (a third product on the same values) run on two streams
+        # dsd's gradients are one launch or two launches on two streams, those of the dds (a third product on the same
+        # values) run on two streams
         return stk.ops.dsd(h, w2s), stk.ops.dds(a, h)
 
     def step():

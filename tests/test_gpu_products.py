@@ -680,7 +680,7 @@ def test_both_gradients_of_dsd_in_one_call(dtype, blocking, hidden, ffn, tokens,
     # through autograd: the gradients of dsd with the joint call and with two launches
     grads = {}
     for joint in (True, False):
-        monkeypatch.setattr(autograd, "JOINT_GRADIENTS", joint)
+        monkeypatch.setattr(autograd, "JOINT_DSD_GRADIENTS", joint)
         ss, rs = s.detach().clone().requires_grad_(True), rhs.detach().clone().requires_grad_(True)
         m = stk.Matrix(tm.size(), ss, tm.row_indices, tm.column_indices, tm.offsets, tm.column_indices_t, tm.offsets_t, tm.block_offsets_t)
         stk.ops.dsd(m.t() if transpose_a else m, rs).backward(dy)
