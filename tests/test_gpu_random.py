@@ -123,6 +123,7 @@ def test_random_products_and_gradients_against_dense_fp32(batch):
 
 def _same(name, got, want, info):
     got = got.cpu().numpy() if torch.is_tensor(got) else np.asarray(got)
+    want = want.cpu().numpy() if torch.is_tensor(want) else want
     assert got.shape == np.asarray(want).shape and np.array_equal(got, want), (name, info)
 
 
@@ -167,3 +168,68 @@ def test_random_routings_and_formats_bit_exact_against_the_oracle(batch):
             _same("to_sparse " + f, getattr(s, f), getattr(wt, f), info)
         _same("to_dense", stk.ops.to_dense(s), xd, info)
         _same("row_indices", stk.ops.row_indices(s.size(), s.data, s.offsets, s.column_indices), wt.row_indices, info)
+
+
+@pytest.mark.parametrize("batch", range(2))
+def test_random_routed_products_bit_exact_against_the_two_launches(batch):
+    """stk_sdd_gather, stk_dsd_scatter and the sums kept by stk_sdd_fused_sums on random routings and sizes: the
+    products on the token rows must give the bits of copy + product (where the library has no kernel for a case the
+    ops run the two launches, and the comparison holds trivially)."""
+    from stk_amd.backend import hip_kernels
+    fused = {"gather": 0, "scatter": 0}
+    for case in range(12):
+        seed = 9100 + batch * 12 + case
+        rng = np.random.RandomState(seed)
+        torch.manual_seed(seed)
+        dtype = [torch.bfloat16, torch.float16][int(rng.randint(2))]
+        experts = int(rng.choice([2, 5, 8, 16, 33]))
+        top_k = int(rng.choice([1, 1, 2]))
+        tokens = int(rng.choice([300, 1500, 4000, 9000]))
+        hidden = int(rng.choice([128, 256, 384, 512, 1024]))
+        ffn = int(rng.choice([128, 384, 1024, 2560]))
+        skew = float(rng.choice([0.0, 1.5, 4.0]))
+        if case < 2:     # enough blocks x columns for the eight-wavefront dsd, whose store the scatter is part of
+            experts, top_k, tokens, hidden, ffn = 8, 1, 9000, [1024, 512][case], [2560, 5120][case]
+        info = dict(seed=seed, dtype=dtype, experts=experts, top_k=top_k, tokens=tokens, hidden=hidden, ffn=ffn, skew=skew)
+        logits = torch.randn(tokens, experts)
+        logits[:, 0] += skew
+        if experts > 2:
+            logits[:, 1] = -1e9                      # an expert without tokens
+        top = logits.topk(top_k, dim=1).indices.to(torch.int32).to(DEV)
+        capacity = stk.ops.route_capacity(tokens * top_k, experts, 128) if rng.rand() < 0.3 else None
+        r = stk.ops.route(top, experts, 128, padded_rows=capacity)
+        rows = r.row_slots.numel()
+        topo = stk.ops.dmoe_topology(r.padded_bins, 128, rows // 128, ffn // 128, dtype=dtype)
+        x = torch.randn(tokens, hidden).to(dtype).to(DEV)
+        w1 = (torch.randn(hidden, experts * ffn) * 0.05).to(dtype).to(DEV)
+        w2 = (torch.randn(experts * ffn, hidden) * 0.05).to(dtype).to(DEV)
+        if rng.rand() < 0.5:
+            w1 = w1.t().contiguous().t()
+        if rng.rand() < 0.5:
+            w2 = w2.t().contiguous().t()
+        activation = [None, "relu", "gelu_tanh", "silu"][int(rng.randint(4))]
+        weights = (torch.rand(tokens, top_k, device=DEV) + 0.5) if rng.rand() < 0.5 else None
+        padded = stk.ops.padded_gather(x, r)
+        want_h = stk.ops.sdd_fused(padded, w1, topo, activation)
+        got_h = stk.ops.gather_sdd(x, r, w1, topo, activation)
+        _same("gather_sdd", got_h.data.view(torch.int16), want_h.data.view(torch.int16), info)
+        want_y = stk.ops.padded_scatter(stk.ops.dsd(want_h, w2), r, weights)
+        got_y = stk.ops.dsd_scatter(want_h, w2, r, weights)
+        _same("dsd_scatter", got_y.view(torch.int16), want_y.view(torch.int16), info)
+        # which cases reached the kernels
+        out = torch.empty_like(topo.data)
+        fused["gather"] += bool(hip_kernels.sdd_gather(x, r.row_slots, top_k, w1, topo.size(), out, topo.offsets, topo.row_indices,
+                                                       topo.column_indices, activation))
+        if top_k == 1:
+            y = torch.empty(tokens, hidden, dtype=dtype, device=DEV)
+            fused["scatter"] += bool(hip_kernels.dsd_scatter(want_h.size(), want_h.data, want_h.offsets, want_h.column_indices, want_h.offsets_t,
+                                                             want_h.column_indices_t, w2, r.row_slots, weights, y))
+        # the kept sums are the plain product
+        if activation is not None:
+            sums = torch.empty_like(topo.data)
+            again = torch.empty_like(topo.data)
+            hip_kernels.sdd_fused(padded, w1, topo.size(), again, topo.offsets, topo.row_indices, topo.column_indices, activation, sums=sums)
+            _same("sums", sums.view(torch.int16), stk.ops.sdd(padded, w1, topo).data.view(torch.int16), info)
+            _same("fused beside sums", again.view(torch.int16), want_h.data.view(torch.int16), info)
+    assert fused["gather"] >= 8, fused     # every case at blocking 128 has the gathered product
+    assert fused["scatter"] >= 2, fused
