@@ -15,6 +15,7 @@ the reference's plumbing configuration - products on CPU tensors - runs here.
 """
 import ctypes
 import threading
+import time
 
 import torch
 
@@ -579,7 +580,7 @@ def to_dense(data, row_indices, column_indices, rows, cols):
     return out
 
 
-NNZ_POLL_LIMIT = 200000   # polls of the pinned nnz word (some 20 ms) before to_sparse waits for the stream instead
+NNZ_POLL_LIMIT = 20000   # polls of the pinned nnz word (some 2 ms) before to_sparse waits for the stream instead
 _nnz_buffers = threading.local()   # per host thread: device index -> pinned int32[1] that stk_to_sparse_count_nnz writes nnz into
 
 
@@ -627,6 +628,8 @@ def to_sparse(x, blocking, index_dtype=torch.int16):
         spins = 0
         while word[0] < 0 and spins < NNZ_POLL_LIMIT:
             spins += 1
+            if not spins & 1023:
+                time.sleep(0)   # let other host threads have the interpreter
         if word[0] < 0:
             torch.cuda.current_stream(dev).synchronize()
             assert word[0] >= 0, "stk_to_sparse_count_nnz did not deliver nnz"
