@@ -675,6 +675,13 @@ __device__ __forceinline__ void mainloop_reg(f32x16_t (&acc)[Cfg::IM][Cfg::JN], 
   }
 }
 
+// Where row m of a 64-row staging quadrant (rows of 128 bytes) keeps its pieces: bits 0-2 are XOR-ed into the index of
+// the 16-byte piece, bit 3 swaps the two 8-byte halves of a piece.  A staging write (64 lanes x 8 bytes: rows m ..
+// m + 31 of one piece column, both halves) then touches every bank once per 16 lanes whether the banks repeat every 128
+// or every 256 bytes: 16 consecutive rows get 16 different (piece, half) places, and the rows 16 apart, which share
+// a place, differ in the parity that selects the upper or lower 128 bytes of a 256-byte bank row.
+__device__ __forceinline__ int staging_swizzle(int m) { return (m ^ ((m >> 4) & 1)) & 15; }
+
 // Writes the wavefront's part of the workgroup tile.  `out` points at element
 // (0, 0) of the wavefront's sub-tile, ldc in elements; rows >= m_valid and
 // columns >= n_valid (both relative to `out`, n_valid a multiple of 8) are
@@ -714,7 +721,7 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   if constexpr (Cfg::WK == 1) {
-    char* s = smem + wave * 8192;  // [64 m][64 n] 16-bit, rows of 128 bytes, 8-byte units swizzled by the row
+    char* s = smem + wave * 8192;  // [64 m][64 n] 16-bit, rows of 128 bytes, 8-byte units swizzled by the row (staging_swizzle)
 #pragma unroll
     for (int qi = 0; qi < (Cfg::IM + 1) / 2; qi++)
 #pragma unroll
@@ -767,7 +774,8 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
                 int m = i * 32 + (lane & 31);
                 int ch = 4 * j + g;
                 u32x2 v = {pack2<Cfg::BF16>(c[4 * g], c[4 * g + 1]), pack2<Cfg::BF16>(c[4 * g + 2], c[4 * g + 3])};
-                *reinterpret_cast<u32x2*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4) + ((((lane >> 5) ^ (m >> 4)) & 1) << 3)) = v;
+                const int sw = staging_swizzle(m);
+                *reinterpret_cast<u32x2*>(s + m * 128 + ((ch ^ (sw & 7)) << 4) + ((((lane >> 5) ^ (sw >> 3)) & 1) << 3)) = v;
               }
         };
         // piece `it` of the staged pass: eight consecutive elements of a row
@@ -775,8 +783,9 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[Cfg::IM][Cfg::JN], elem
         auto staged = [&](int it) {
           int m = it * 8 + (lane >> 3);
           int ch = lane & 7;
-          u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ ((m >> 1) & 7)) << 4));
-          if ((m >> 4) & 1) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
+          const int sw = staging_swizzle(m);
+          u32x4 v = *reinterpret_cast<const u32x4*>(s + m * 128 + ((ch ^ (sw & 7)) << 4));
+          if (sw >> 3) v = u32x4{v.z, v.w, v.x, v.y};  // the two 8-byte halves were stored swapped
           return v;
         };
         if (sums) {
